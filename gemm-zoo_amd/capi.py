@@ -1,0 +1,142 @@
+"""ctypes binding of ``lib/libgemmzoo.so`` (the C ABI declared in ``include/gemm_zoo.h``).
+
+The library is the only compute path: if it is missing this module raises at import
+time instead of falling back to anything else.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+_HERE = Path(__file__).resolve().parent
+LIB_PATH = _HERE / "lib" / "libgemmzoo.so"
+
+# enums of include/gemm_zoo.h
+OK, ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_MISMATCH = 0, 1, 2, 3, 4
+ROW_MAJOR, COL_MAJOR = 0, 1
+S8S8S32, BF16BF16F32, BF16BF16BF16, F16F16F16 = 0, 1, 2, 3
+RUNG_AUTO, RUNG_NAIVE, RUNG_COALESCED, RUNG_LDS_TILED, RUNG_DOUBLE_BUFFERED, RUNG_MFMA, RUNG_SKINNY = -1, 0, 1, 2, 3, 4, 5
+NUM_RUNGS = 6
+DT_INT8, DT_BF16, DT_F16, DT_F32, DT_INT32 = 0, 1, 2, 3, 4
+FILL_INT8_UNIFORM, FILL_NORMAL, FILL_UNIFORM_PM1, FILL_SMALL_INT = 0, 1, 2, 3
+
+TYPES_NAMES = {S8S8S32: "s8s8s32", BF16BF16F32: "bf16bf16f32", BF16BF16BF16: "bf16bf16bf16", F16F16F16: "f16f16f16"}
+IN_SIZE = {S8S8S32: 1, BF16BF16F32: 2, BF16BF16BF16: 2, F16F16F16: 2}
+OUT_SIZE = {S8S8S32: 4, BF16BF16F32: 4, BF16BF16BF16: 2, F16F16F16: 2}
+
+EXPORTS = [
+    "gz_gemm_s8s8s32", "gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16", "gz_gemm",
+    "gz_plan", "gz_variant_count", "gz_rung_name", "gz_types_name", "gz_fill", "gz_compare",
+    "gz_last_error", "gz_version",
+]
+
+
+class GzError(RuntimeError):
+    """A non-zero gz_status; ``status`` holds the code, the text is gz_last_error()."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"gz status {status}: {message}")
+        self.status = status
+
+
+class Plan(C.Structure):
+    _fields_ = [
+        ("rung", C.c_int32), ("variant", C.c_int32),
+        ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
+        ("wave_m", C.c_int32), ("wave_n", C.c_int32),
+        ("threads", C.c_int32), ("lds_bytes", C.c_int32),
+        ("grid", C.c_int64), ("split_k", C.c_int32),
+        ("vector_bytes_a", C.c_int32), ("vector_bytes_b", C.c_int32),
+    ]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+def _load():
+    if not LIB_PATH.exists():
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python gemm-zoo_amd/build.py` "
+            "(there is no fallback path)")
+    lib = C.CDLL(str(LIB_PATH))
+    vp, i64, i32, f32, f64 = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_double
+    common = [vp, vp, vp, vp, i64, i64, i64, i32, i32]
+    lib.gz_gemm_s8s8s32.argtypes = common + [C.c_int32, C.c_int32, i32, i32, vp]
+    for name in ("gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16"):
+        getattr(lib, name).argtypes = common + [f32, f32, i32, i32, vp]
+    lib.gz_gemm.argtypes = [i32] + common + [f64, f64, i32, i32, vp]
+    lib.gz_plan.argtypes = [i32, i64, i64, i64, i32, i32, i32, i32, i32, i32, C.POINTER(Plan)]
+    lib.gz_variant_count.argtypes = [i32, i32]
+    lib.gz_rung_name.argtypes = [i32]
+    lib.gz_rung_name.restype = C.c_char_p
+    lib.gz_types_name.argtypes = [i32]
+    lib.gz_types_name.restype = C.c_char_p
+    lib.gz_fill.argtypes = [vp, i64, i32, i32, f32, C.c_uint64, vp]
+    lib.gz_compare.argtypes = [vp, vp, i64, i32, f32, C.POINTER(C.c_int64), vp]
+    lib.gz_last_error.restype = C.c_char_p
+    for name in EXPORTS:
+        fn = getattr(lib, name)
+        if fn.restype is C.c_int or fn.restype is None:
+            fn.restype = C.c_int
+    return lib
+
+
+lib = _load()
+
+
+def last_error() -> str:
+    return lib.gz_last_error().decode()
+
+
+def check(status: int) -> None:
+    if status != OK:
+        raise GzError(status, last_error())
+
+
+def _ptr(x) -> int:
+    """Device pointer of a torch tensor, an int, or None."""
+    if x is None:
+        return 0
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()
+
+
+def gemm(types: int, a, b, c, d, m: int, n: int, k: int, layout_a: int = ROW_MAJOR, layout_b: int = ROW_MAJOR,
+         alpha=1, beta=0, rung: int = RUNG_AUTO, variant: int = 0, stream: int = 0) -> None:
+    """Typed entry point dispatch (raises GzError on a non-zero status)."""
+    fn = {S8S8S32: lib.gz_gemm_s8s8s32, BF16BF16F32: lib.gz_gemm_bf16bf16f32,
+          BF16BF16BF16: lib.gz_gemm_bf16bf16bf16, F16F16F16: lib.gz_gemm_f16f16f16}.get(types)
+    if fn is None:
+        raise GzError(ERR_BAD_ARG, f"unknown type bundle {types}")
+    if types == S8S8S32:
+        alpha, beta = int(alpha), int(beta)
+    check(fn(_ptr(a), _ptr(b), _ptr(c), _ptr(d), m, n, k, layout_a, layout_b, alpha, beta, rung, variant, stream))
+
+
+def plan(types: int, m: int, n: int, k: int, layout_a: int = ROW_MAJOR, layout_b: int = ROW_MAJOR,
+         rung: int = RUNG_AUTO, variant: int = 0, num_cus: int = 0, lds_per_cu: int = 0) -> Plan:
+    p = Plan()
+    check(lib.gz_plan(types, m, n, k, layout_a, layout_b, rung, variant, num_cus, lds_per_cu, C.byref(p)))
+    return p
+
+
+def fill(dst, count: int, dtype: int, kind: int, scale: float = 1.0, seed: int = 2025, stream: int = 0) -> None:
+    check(lib.gz_fill(_ptr(dst), count, dtype, kind, scale, seed, stream))
+
+
+def compare(out, ref, count: int, dtype: int, abs_threshold: float = 0.0, stream: int = 0) -> int:
+    """Returns the number of differing elements (0 = equal); raises only on API errors."""
+    nd = C.c_int64(0)
+    st = lib.gz_compare(_ptr(out), _ptr(ref), count, dtype, abs_threshold, C.byref(nd), stream)
+    if st not in (OK, ERR_MISMATCH):
+        raise GzError(st, last_error())
+    return nd.value
+
+
+def variant_count(types: int, rung: int) -> int:
+    return lib.gz_variant_count(types, rung)
+
+
+def rung_name(rung: int) -> str:
+    return lib.gz_rung_name(rung).decode()

@@ -1,0 +1,260 @@
+// extern "C" layer: argument checks, rung dispatch, launch planning, error text.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <cmath>
+
+#include "gz_common.hpp"
+#include "gz_mfma_cfg.hpp"
+#include "gz_skinny_cfg.hpp"
+
+namespace gz {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  set_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+  return GZ_ERR_HIP;
+}
+
+static const char* kRungNames[GZ_NUM_RUNGS] = {"naive", "coalesced", "lds_tiled", "double_buffered", "mfma", "skinny"};
+static const char* kTypesNames[4] = {"s8s8s32", "bf16bf16f32", "bf16bf16bf16", "f16f16f16"};
+
+static int in_size(int types) { return types == GZ_S8S8S32 ? 1 : 2; }
+static int out_size(int types) { return (types == GZ_S8S8S32 || types == GZ_BF16BF16F32) ? 4 : 2; }
+
+// Shape / enum checks common to gz_plan and the GEMM entry points.
+static int check_problem(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung) {
+  if (types < 0 || types > 3) {
+    set_error("unknown type bundle %d", types);
+    return GZ_ERR_BAD_ARG;
+  }
+  if (M < 0 || N < 0 || K < 0) {
+    set_error("negative size M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    return GZ_ERR_BAD_ARG;
+  }
+  if ((layoutA != GZ_ROW_MAJOR && layoutA != GZ_COL_MAJOR) || (layoutB != GZ_ROW_MAJOR && layoutB != GZ_COL_MAJOR)) {
+    set_error("unknown layout A=%d B=%d", layoutA, layoutB);
+    return GZ_ERR_BAD_ARG;
+  }
+  if (rung < GZ_RUNG_AUTO || rung >= GZ_NUM_RUNGS) {
+    set_error("unknown rung %d", rung);
+    return GZ_ERR_BAD_ARG;
+  }
+  // kernels index with 32-bit element counts per matrix
+  const int64_t lim = (int64_t)1 << 31;
+  if (M >= lim || N >= lim || K >= lim || M * K >= lim || K * N >= lim || M * N >= lim) {
+    set_error("matrix with 2^31 or more elements is not supported (M=%lld N=%lld K=%lld)", (long long)M,
+              (long long)N, (long long)K);
+    return GZ_ERR_UNSUPPORTED;
+  }
+  return GZ_OK;
+}
+
+static int resolve_rung(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung) {
+  if (rung != GZ_RUNG_AUTO) return rung;
+  if (skinny_supported(types, (int)M, (int)N, (int)K, layoutA, layoutB)) return GZ_RUNG_SKINNY;
+  return GZ_RUNG_MFMA;
+}
+
+template <int TYPES>
+static int run(const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K, int layoutA,
+               int layoutB, typename Traits<TYPES>::scalar_t alpha, typename Traits<TYPES>::scalar_t beta, int rung,
+               int variant, gz_stream stream) {
+  using T = Traits<TYPES>;
+  int st = check_problem(TYPES, M, N, K, layoutA, layoutB, rung);
+  if (st != GZ_OK) return st;
+  if (M == 0 || N == 0) return GZ_OK;  // nothing to write
+  if (!A && K > 0 && M > 0) { set_error("A is NULL"); return GZ_ERR_BAD_ARG; }
+  if (!B && K > 0 && N > 0) { set_error("B is NULL"); return GZ_ERR_BAD_ARG; }
+  if (!D) { set_error("D is NULL"); return GZ_ERR_BAD_ARG; }
+  if (!C && beta != 0) { set_error("C is NULL but beta != 0"); return GZ_ERR_BAD_ARG; }
+  if (variant < 0) { set_error("negative variant %d", variant); return GZ_ERR_BAD_ARG; }
+
+  GemmArgs<TYPES> g;
+  g.A = static_cast<const typename T::in_t*>(A);
+  g.B = static_cast<const typename T::in_t*>(B);
+  g.C = static_cast<const typename T::out_t*>(C);
+  g.D = static_cast<typename T::out_t*>(D);
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.layoutA = layoutA; g.layoutB = layoutB;
+  g.alpha = alpha; g.beta = beta;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  switch (resolve_rung(TYPES, M, N, K, layoutA, layoutB, rung)) {
+    case GZ_RUNG_NAIVE: return launch_naive<TYPES>(g, variant, s);
+    case GZ_RUNG_COALESCED: return launch_coalesced<TYPES>(g, variant, s);
+    case GZ_RUNG_LDS_TILED: return launch_lds_tiled<TYPES>(g, variant, s);
+    case GZ_RUNG_DOUBLE_BUFFERED: return launch_double_buffered<TYPES>(g, variant, s);
+    case GZ_RUNG_MFMA: return launch_mfma<TYPES>(g, variant, s);
+    case GZ_RUNG_SKINNY: return launch_skinny<TYPES>(g, variant, s);
+    default: break;
+  }
+  set_error("unknown rung %d", rung);
+  return GZ_ERR_BAD_ARG;
+}
+
+}  // namespace gz
+
+using namespace gz;
+
+extern "C" {
+
+int gz_gemm_s8s8s32(const int8_t* A, const int8_t* B, const int32_t* C, int32_t* D, int64_t M, int64_t N, int64_t K,
+                    int layoutA, int layoutB, int32_t alpha, int32_t beta, int rung, int variant, gz_stream stream) {
+  return run<GZ_S8S8S32>(A, B, C, D, M, N, K, layoutA, layoutB, alpha, beta, rung, variant, stream);
+}
+
+int gz_gemm_bf16bf16f32(const uint16_t* A, const uint16_t* B, const float* C, float* D, int64_t M, int64_t N,
+                        int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung, int variant,
+                        gz_stream stream) {
+  return run<GZ_BF16BF16F32>(A, B, C, D, M, N, K, layoutA, layoutB, alpha, beta, rung, variant, stream);
+}
+
+int gz_gemm_bf16bf16bf16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int64_t M, int64_t N,
+                         int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung, int variant,
+                         gz_stream stream) {
+  return run<GZ_BF16BF16BF16>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<GZ_BF16BF16BF16>(alpha),
+                              round_out<GZ_BF16BF16BF16>(beta), rung, variant, stream);
+}
+
+int gz_gemm_f16f16f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int64_t M, int64_t N,
+                      int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung, int variant,
+                      gz_stream stream) {
+  return run<GZ_F16F16F16>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<GZ_F16F16F16>(alpha),
+                           round_out<GZ_F16F16F16>(beta), rung, variant, stream);
+}
+
+int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K,
+            int layoutA, int layoutB, double alpha, double beta, int rung, int variant, gz_stream stream) {
+  switch (types) {
+    case GZ_S8S8S32:
+      if (alpha != std::floor(alpha) || beta != std::floor(beta) || std::fabs(alpha) > 2147483647.0 ||
+          std::fabs(beta) > 2147483647.0) {
+        set_error("s8s8s32 needs integral alpha/beta that fit int32");
+        return GZ_ERR_BAD_ARG;
+      }
+      return gz_gemm_s8s8s32((const int8_t*)A, (const int8_t*)B, (const int32_t*)C, (int32_t*)D, M, N, K, layoutA,
+                             layoutB, (int32_t)alpha, (int32_t)beta, rung, variant, stream);
+    case GZ_BF16BF16F32:
+      return gz_gemm_bf16bf16f32((const uint16_t*)A, (const uint16_t*)B, (const float*)C, (float*)D, M, N, K, layoutA,
+                                 layoutB, (float)alpha, (float)beta, rung, variant, stream);
+    case GZ_BF16BF16BF16:
+      return gz_gemm_bf16bf16bf16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
+                                  layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
+    case GZ_F16F16F16:
+      return gz_gemm_f16f16f16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
+                               layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
+    default: break;
+  }
+  set_error("unknown type bundle %d", types);
+  return GZ_ERR_BAD_ARG;
+}
+
+int gz_variant_count(int types, int rung) {
+  if (types < 0 || types > 3) return 0;
+  switch (rung) {
+    case GZ_RUNG_NAIVE: case GZ_RUNG_COALESCED: case GZ_RUNG_LDS_TILED: case GZ_RUNG_DOUBLE_BUFFERED: return 1;
+    case GZ_RUNG_MFMA: return kNumMfmaCfgs;
+    case GZ_RUNG_SKINNY: return types == GZ_S8S8S32 ? 0 : 1;
+    default: return 0;
+  }
+}
+
+int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung, int variant, int num_cus,
+            int lds_per_cu, gz_plan_t* plan) {
+  if (!plan) { set_error("plan is NULL"); return GZ_ERR_BAD_ARG; }
+  int st = check_problem(types, M, N, K, layoutA, layoutB, rung);
+  if (st != GZ_OK) return st;
+  if (variant < 0) { set_error("negative variant %d", variant); return GZ_ERR_BAD_ARG; }
+  if (num_cus <= 0) num_cus = 256;
+  if (lds_per_cu <= 0) lds_per_cu = 160 * 1024;
+  memset(plan, 0, sizeof(*plan));
+  const int r = resolve_rung(types, M, N, K, layoutA, layoutB, rung);
+  plan->rung = r;
+  plan->split_k = 1;
+  const int es = in_size(types);
+  const int m = (int)M, n = (int)N, k = (int)K;
+  const bool a_kc = layoutA == GZ_ROW_MAJOR, b_kc = layoutB == GZ_COL_MAJOR;
+  // widest naturally aligned vector each operand allows (packed lines, 16-byte aligned base assumed)
+  auto vec_bytes = [&](int extent) {
+    int bytes = extent * es, v = 16;
+    while (v > es && bytes % v) v >>= 1;
+    return v;
+  };
+  plan->vector_bytes_a = vec_bytes(a_kc ? k : m);
+  plan->vector_bytes_b = vec_bytes(b_kc ? k : n);
+  switch (r) {
+    case GZ_RUNG_NAIVE:
+      if (variant != 0) { set_error("naive rung has a single variant"); return GZ_ERR_UNSUPPORTED; }
+      plan->tile_m = 32; plan->tile_n = 32; plan->tile_k = 1; plan->threads = 1024;
+      plan->grid = (int64_t)ceil_div(m, 32) * ceil_div(n, 32);
+      plan->vector_bytes_a = plan->vector_bytes_b = es;
+      return GZ_OK;
+    case GZ_RUNG_COALESCED:
+      if (variant != 0) { set_error("coalesced rung has a single variant"); return GZ_ERR_UNSUPPORTED; }
+      plan->tile_m = 16; plan->tile_n = 64; plan->tile_k = 16 / es; plan->threads = 256;
+      plan->grid = (int64_t)ceil_div(m, 16) * ceil_div(n, 64);
+      return GZ_OK;
+    case GZ_RUNG_LDS_TILED:
+    case GZ_RUNG_DOUBLE_BUFFERED: {
+      if (variant != 0) { set_error("rung has a single variant"); return GZ_ERR_UNSUPPORTED; }
+      const int stages = r == GZ_RUNG_DOUBLE_BUFFERED ? 2 : 1;
+      plan->tile_m = 64; plan->tile_n = 64; plan->tile_k = 32; plan->threads = 256;
+      plan->lds_bytes = stages * 2 * 32 * (64 + 4) * 4;
+      plan->grid = (int64_t)ceil_div(m, 64) * ceil_div(n, 64);
+      return GZ_OK;
+    }
+    case GZ_RUNG_MFMA: {
+      MfmaCfg c;
+      if (!mfma_resolve(types, m, n, k, variant, num_cus, &c)) {
+        set_error("mfma rung: unknown variant %d", variant);
+        return GZ_ERR_UNSUPPORTED;
+      }
+      plan->variant = c.id;
+      plan->tile_m = c.bm; plan->tile_n = c.bn; plan->tile_k = MFMA_SLAB_BYTES / es;
+      plan->wave_m = c.bm / c.waves_m; plan->wave_n = c.bn / c.waves_n;
+      plan->threads = c.waves_m * c.waves_n * 64;
+      plan->lds_bytes = mfma_lds_bytes(c);
+      plan->grid = (int64_t)ceil_div(m, c.bm) * ceil_div(n, c.bn);
+      if (plan->lds_bytes > lds_per_cu) {
+        set_error("mfma variant %d needs %d bytes of LDS, device has %d", c.id, plan->lds_bytes, lds_per_cu);
+        return GZ_ERR_UNSUPPORTED;
+      }
+      return GZ_OK;
+    }
+    case GZ_RUNG_SKINNY: {
+      if (!skinny_supported(types, m, n, k, layoutA, layoutB)) {
+        set_error("skinny rung needs a 16-bit float type, row-major A, column-major B, M <= %d and K %% 8 == 0",
+                  SKINNY_MAX_M);
+        return GZ_ERR_UNSUPPORTED;
+      }
+      if (variant > 1) { set_error("skinny rung has a single variant"); return GZ_ERR_UNSUPPORTED; }
+      SkinnyCfg c = skinny_resolve(m, n, k, num_cus);
+      plan->variant = 1;
+      plan->tile_m = c.mb; plan->tile_n = c.cols_per_wg; plan->tile_k = c.k_per_split;
+      plan->wave_m = c.mb; plan->wave_n = c.cols_per_wave;
+      plan->threads = c.threads; plan->split_k = c.split_k;
+      plan->grid = (int64_t)c.grid_n * c.split_k;
+      return GZ_OK;
+    }
+    default: break;
+  }
+  set_error("unknown rung %d", rung);
+  return GZ_ERR_BAD_ARG;
+}
+
+const char* gz_rung_name(int rung) { return (rung >= 0 && rung < GZ_NUM_RUNGS) ? kRungNames[rung] : "auto"; }
+const char* gz_types_name(int types) { return (types >= 0 && types < 4) ? kTypesNames[types] : "?"; }
+const char* gz_last_error(void) { return g_err; }
+int gz_version(void) { return 1; }
+
+}  // extern "C"

@@ -1,0 +1,57 @@
+// Host-side tile-config table of the MFMA rung (shared by the launcher and gz_plan).
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+namespace gz {
+
+struct MfmaCfg {
+  int id;       // variant id (1-based; 0 means "let the launcher choose")
+  int bm, bn;   // work-group tile
+  int waves_m, waves_n;
+};
+
+// K slab per tile row is 128 bytes whatever the element type.
+constexpr int MFMA_SLAB_BYTES = 128;
+constexpr int MFMA_LDS_PITCH = 144;
+
+static const MfmaCfg kMfmaCfgs[] = {
+    {1, 256, 256, 2, 2},  // 4 waves of 128x128: fewest LDS bytes per MFMA
+    {2, 256, 256, 2, 4},  // 8 waves of 128x64: two waves per SIMD hide each other's waits
+    {3, 128, 128, 2, 2},  // small tile for small problems / ragged tails
+    {4, 256, 128, 2, 2},  // 4 waves of 128x64
+};
+constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
+
+inline int mfma_lds_bytes(const MfmaCfg& c) { return 2 * (c.bm + c.bn) * MFMA_LDS_PITCH; }
+
+// Picks the tile configuration.  A 256x256 tile needs the fewest bytes per flop;
+// it is kept as long as the grid still covers every compute unit, otherwise the
+// tile shrinks so that more work-groups exist.
+inline bool mfma_resolve(int /*types*/, int M, int N, int /*K*/, int variant, int num_cus, MfmaCfg* out) {
+  if (variant < 0 || variant > kNumMfmaCfgs) return false;
+  if (variant > 0) {
+    *out = kMfmaCfgs[variant - 1];
+    return true;
+  }
+  auto tiles = [&](const MfmaCfg& c) {
+    return (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  };
+  if (tiles(kMfmaCfgs[0]) >= num_cus) *out = kMfmaCfgs[0];
+  else if (tiles(kMfmaCfgs[3]) >= num_cus) *out = kMfmaCfgs[3];
+  else *out = kMfmaCfgs[2];
+  return true;
+}
+
+// The unpredicated kernel needs whole tiles, whole K slabs and 16-byte aligned
+// operands; everything else runs the predicated (edge) instantiation.
+inline bool mfma_needs_edge(const MfmaCfg& c, int in_size, int /*out_size*/, int M, int N, int K, const void* A,
+                            const void* B, const void* C, const void* D) {
+  const int bk = MFMA_SLAB_BYTES / in_size;
+  if (K == 0 || M % c.bm || N % c.bn || K % bk) return true;
+  const uintptr_t bits = (uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)D;
+  return (bits & 15u) != 0;
+}
+
+}  // namespace gz

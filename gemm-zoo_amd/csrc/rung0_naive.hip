@@ -1,0 +1,52 @@
+// Rung 0: one thread per output element, scalar loads, sequential k.
+// Follows the definition of the operation in gemm-zoo
+// (nvidia/kernels/naive_gemm.cuh:6-21, intel/utils/reference_kernel.hpp:12-28),
+// generalised to column-major operands; the accumulator is fp32 / int32.
+#include "gz_common.hpp"
+
+namespace gz {
+
+template <int TYPES, bool A_ROW, bool B_ROW>
+__global__ void __launch_bounds__(1024) naive_gemm_kernel(GemmArgs<TYPES> g) {
+  using T = Traits<TYPES>;
+  const int col = threadIdx.x + blockIdx.x * blockDim.x;
+  const int row = threadIdx.y + blockIdx.y * blockDim.y;
+  if (row >= g.M || col >= g.N) return;
+
+  typename T::acc_t acc = 0;
+  for (int i = 0; i < g.K; i++) {
+    const auto a = widen_in<TYPES>(A_ROW ? g.A[(size_t)row * g.K + i] : g.A[(size_t)i * g.M + row]);
+    const auto b = widen_in<TYPES>(B_ROW ? g.B[(size_t)i * g.N + col] : g.B[(size_t)col * g.K + i]);
+    if constexpr (T::is_int) acc += a * b;
+    else acc = __builtin_fmaf(a, b, acc);  // a*b is exact in fp32 for 16-bit inputs
+  }
+  const size_t o = (size_t)row * g.N + col;
+  g.D[o] = epilogue<TYPES>(acc, g.alpha, g.beta, g.C + o);
+}
+
+template <int TYPES> int launch_naive(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
+  if (variant != 0) {
+    set_error("naive rung has a single variant (got %d)", variant);
+    return GZ_ERR_UNSUPPORTED;
+  }
+  dim3 block(32, 32, 1);  // nvidia/kernel_functors/naive_gemm.cuh:15-16
+  dim3 grid(ceil_div(g.N, 32), ceil_div(g.M, 32), 1);
+  if (grid.y > 65535u) {
+    set_error("naive rung: M=%d needs more than 65535 block rows", g.M);
+    return GZ_ERR_UNSUPPORTED;
+  }
+  const bool ar = g.layoutA == GZ_ROW_MAJOR, br = g.layoutB == GZ_ROW_MAJOR;
+  if (ar && br) hipLaunchKernelGGL((naive_gemm_kernel<TYPES, true, true>), grid, block, 0, s, g);
+  else if (ar && !br) hipLaunchKernelGGL((naive_gemm_kernel<TYPES, true, false>), grid, block, 0, s, g);
+  else if (!ar && br) hipLaunchKernelGGL((naive_gemm_kernel<TYPES, false, true>), grid, block, 0, s, g);
+  else hipLaunchKernelGGL((naive_gemm_kernel<TYPES, false, false>), grid, block, 0, s, g);
+  GZ_HIP_TRY(hipGetLastError());
+  return GZ_OK;
+}
+
+template int launch_naive<GZ_S8S8S32>(const GemmArgs<GZ_S8S8S32>&, int, hipStream_t);
+template int launch_naive<GZ_BF16BF16F32>(const GemmArgs<GZ_BF16BF16F32>&, int, hipStream_t);
+template int launch_naive<GZ_BF16BF16BF16>(const GemmArgs<GZ_BF16BF16BF16>&, int, hipStream_t);
+template int launch_naive<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hipStream_t);
+
+}  // namespace gz

@@ -1,0 +1,152 @@
+/*
+ * gemm_zoo.h -- C ABI of the MI355X (gfx950) GEMM kernel ladder.
+ *
+ * D = alpha * (A x B) + beta * C   with A: M x K, B: K x N, C and D: M x N.
+ *
+ * All matrix pointers are DEVICE pointers owned by the caller, packed (the
+ * leading dimension equals the contiguous extent).  C and D are always
+ * row-major.  A and B carry a layout flag each.  When beta == 0, C is never
+ * read and may be NULL.  D must not overlap A or B.  Calls are asynchronous on
+ * `stream` (a hipStream_t, NULL = the default stream); the caller synchronises.
+ *
+ * Every function returns a gz_status; nothing exits the process or throws.
+ * gz_last_error() gives the message of the calling thread's last failure.
+ *
+ * What each entry point stands in for in gemm-zoo (paths relative to its tree):
+ *   typed GEMM entry points  <-  the kernel functors' operator()
+ *       nvidia/kernel_functors/bf16_mma_gemm.cuh:51-63   (bf16 x bf16 -> f32)
+ *       nvidia/kernel_functors/fp16_mma_gemm.cuh:16-70   (fp16 x fp16 -> fp16)
+ *       intel/xe_gemm_s8_s8_s32_m8k16.hpp:12-40          (s8 x s8 -> s32)
+ *       intel/xe_gemm_bf16_bf16_f32_m8k16.hpp:12-47      (bf16 x bf16 -> f32)
+ *       intel/xe_gemm_bf16_bf16_bf16_m8k16.hpp:12-47     (bf16 x bf16 -> bf16)
+ *       nvidia/kernel_functors/naive_gemm.cuh:12-31, generic_gemm.cuh:14-41,
+ *       smem_tiled_gemm.cuh:14-51, rmem_tiled_gemm.cuh:15-55,
+ *       double_buffered_gemm.cuh:15-57, async_buffered_gemm.cuh:16-58 (ladder rungs)
+ *   gz_plan                   <-  the functors' constructors (grid/block/LDS
+ *       computation and shape checks), e.g. nvidia/kernel_functors/bf16_mma_gemm.cuh:18-49
+ *   gz_fill                   <-  utils::populate_with_random nvidia/utils/fill_data.cuh:33-49,
+ *                                 test::populate_with_random intel/test/utils.hpp:27-45
+ *   gz_compare                <-  utils::compare_results nvidia/utils/compare.cuh:32-47,
+ *                                 test::compare_results intel/test/utils.hpp:47-73
+ *
+ * Arithmetic contract (what the parity tests hold the kernels to):
+ *   s8s8s32     : int32 accumulate, D = alpha*acc + beta*C in wrapping int32.
+ *   bf16bf16f32 : fp32 accumulate, v = acc*alpha; if (beta != 0) v += beta*C; each
+ *                 operation rounded to fp32 (no fused multiply-add in the epilogue).
+ *   bf16bf16bf16, f16f16f16 : fp32 accumulate, then the same epilogue evaluated in the
+ *                 16-bit output type: v = T(acc); v = T(v*alpha); if (beta != 0)
+ *                 v = T(v + T(beta*C)) -- nvidia/kernels/generic_gemm.cuh:53-58.
+ *                 alpha and beta are rounded to the output type first.
+ */
+#ifndef GEMM_ZOO_H
+#define GEMM_ZOO_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum gz_status {
+  GZ_OK = 0,
+  GZ_ERR_BAD_ARG = 1,     /* null pointer, negative size, unknown enum value      */
+  GZ_ERR_UNSUPPORTED = 2, /* valid request this rung / variant cannot serve       */
+  GZ_ERR_HIP = 3,         /* a HIP runtime call failed; see gz_last_error()       */
+  GZ_ERR_MISMATCH = 4     /* gz_compare found differing elements                  */
+} gz_status;
+
+typedef enum gz_layout { GZ_ROW_MAJOR = 0, GZ_COL_MAJOR = 1 } gz_layout;
+
+typedef enum gz_types {
+  GZ_S8S8S32 = 0,
+  GZ_BF16BF16F32 = 1,
+  GZ_BF16BF16BF16 = 2,
+  GZ_F16F16F16 = 3
+} gz_types;
+
+/* The ladder.  GZ_RUNG_AUTO lets the launcher pick (MFMA, or the weight-streaming
+ * kernel for skinny M).                                                            */
+typedef enum gz_rung {
+  GZ_RUNG_AUTO = -1,
+  GZ_RUNG_NAIVE = 0,           /* one thread per output, scalar loads              */
+  GZ_RUNG_COALESCED = 1,       /* layout-aware lane mapping, 128-bit global loads  */
+  GZ_RUNG_LDS_TILED = 2,       /* LDS tiles with bank-conflict-free padding        */
+  GZ_RUNG_DOUBLE_BUFFERED = 3, /* global->LDS prefetch overlapped with compute     */
+  GZ_RUNG_MFMA = 4,            /* wavefront-level matrix-core kernel               */
+  GZ_RUNG_SKINNY = 5,          /* weight-streaming kernel for M <= 128             */
+  GZ_NUM_RUNGS = 6
+} gz_rung;
+
+typedef void* gz_stream; /* hipStream_t */
+
+/* Launch geometry the launcher chose for a problem (host-only computation). */
+typedef struct gz_plan_t {
+  int32_t rung;        /* resolved rung (never GZ_RUNG_AUTO)                   */
+  int32_t variant;     /* resolved tile-config id within the rung              */
+  int32_t tile_m, tile_n, tile_k;
+  int32_t wave_m, wave_n;      /* per-wavefront sub-tile (0 if not applicable) */
+  int32_t threads;             /* work-group size                              */
+  int32_t lds_bytes;           /* static + dynamic LDS per work-group          */
+  int64_t grid;                /* number of work-groups                        */
+  int32_t split_k;             /* >1: partial sums reduced in a second pass    */
+  int32_t vector_bytes_a, vector_bytes_b; /* widest aligned global access used */
+} gz_plan_t;
+
+/* variant: 0 = launcher's choice; other values select a tile configuration of the rung
+ * (see gz_plan / gz_variant_count).                                                  */
+int gz_gemm_s8s8s32(const int8_t* A, const int8_t* B, const int32_t* C, int32_t* D,
+                    int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                    int32_t alpha, int32_t beta, int rung, int variant, gz_stream stream);
+
+int gz_gemm_bf16bf16f32(const uint16_t* A, const uint16_t* B, const float* C, float* D,
+                        int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                        float alpha, float beta, int rung, int variant, gz_stream stream);
+
+int gz_gemm_bf16bf16bf16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                         int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                         float alpha, float beta, int rung, int variant, gz_stream stream);
+
+int gz_gemm_f16f16f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                      int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                      float alpha, float beta, int rung, int variant, gz_stream stream);
+
+/* Type-erased form of the four above (alpha/beta as double; for s8s8s32 they must be
+ * integral).                                                                         */
+int gz_gemm(int types, const void* A, const void* B, const void* C, void* D,
+            int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+            double alpha, double beta, int rung, int variant, gz_stream stream);
+
+/* Host-only: resolve rung/variant and compute the launch geometry for a problem on a
+ * device with `num_cus` compute units and `lds_per_cu` bytes of LDS (0 = MI355X: 256 CUs,
+ * 160 KiB).  Performs the same argument checks as the GEMM entry points.            */
+int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+            int rung, int variant, int num_cus, int lds_per_cu, gz_plan_t* plan);
+
+int gz_variant_count(int types, int rung);
+const char* gz_rung_name(int rung);
+const char* gz_types_name(int types);
+
+/* Seeded device fill: element i of `dst` is a pure function of (seed, i) through
+ * Philox4x32-10 with counter = i and key = seed.
+ *   dtype: 0 int8, 1 bf16, 2 fp16, 3 fp32, 4 int32
+ *   kind : 0 integers uniform in [-128,127]   1 N(0,1)*scale   2 U(-1,1)*scale
+ *          3 small integers in {-1,0,1} (exactly representable partial sums)      */
+int gz_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t seed,
+            gz_stream stream);
+
+/* Element-wise compare of two device arrays.  abs_threshold == 0 demands exact equality
+ * of the stored values; otherwise |out - ref| > abs_threshold counts as different.
+ * Synchronises `stream`.  *num_different (host memory, may be NULL) receives the count.
+ * Returns GZ_ERR_MISMATCH if any element differs.
+ *   dtype as in gz_fill.                                                            */
+int gz_compare(const void* out, const void* ref, int64_t count, int dtype,
+               float abs_threshold, int64_t* num_different, gz_stream stream);
+
+const char* gz_last_error(void);
+int gz_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GEMM_ZOO_H */

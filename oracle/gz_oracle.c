@@ -1,0 +1,531 @@
+/*
+ * gz_oracle.c -- CPU restatement of gemm-zoo's reference GEMM.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is the checker the HIP kernels are
+ * compared against; nothing in the shipped library links, loads or calls it.
+ * Only the test-suite, the smoke check and the "cpu_baseline" leg of the
+ * benchmark may load the shared object built from it.
+ *
+ * What it restates (paths are relative to the reference checkout):
+ *
+ *   - intel/utils/reference_kernel.hpp:12-28  (utils::detail::reference_gemm)
+ *     twin: nvidia/kernels/naive_gemm.cuh:6-21
+ *       one output element per work-item, sequential k from 0, accumulate in
+ *       TOut, then  d = alpha*acc + beta*c.      -> oracle_literal_*()
+ *
+ *   - nvidia/kernels/generic_gemm.cuh:6-60  (nvidia::kernels::generic_gemm)
+ *       inputs cast to float, float sum over k, then
+ *       val = TOut(sum)*alpha; if (beta != 0) val += beta*c   (lines 53-58)
+ *       evaluated in TOut arithmetic.            -> oracle_gemm()
+ *
+ *   - layouts: the reference only knows row-major operands; column-major A/B
+ *     is the generalisation  A(i,p) = rowmajor ? a[i*K+p] : a[p*M+i].
+ *
+ *   - intel/test/utils.hpp:27-45 (populate_with_random): a counter based
+ *     Philox4x32-10 stream keyed by (seed, element_id).  The reference's exact
+ *     streams come from oneMath / cuRAND and cannot be reproduced; only the
+ *     construction (one engine per element, keyed by seed and element index)
+ *     is followed.                               -> oracle_fill_*()
+ *
+ * Pinning (see tests/test_oracle_*.py):
+ *   oracle_literal_*      closed forms (all-ones, identity, single-nonzero
+ *                         probes, extreme int8), brute force vs Python ints.
+ *   oracle_gemm           bit-equal to oracle_literal_* on row-major inputs
+ *                         for s8->s32 and for integer-valued float inputs;
+ *                         fp64 truth within fp32 accumulation bounds; layout
+ *                         probes; beta==0 never reads C.
+ *   bf16/fp16 converters  closed-form RNE known answers, exhaustive 2^16
+ *                         round trips, numpy float16 / torch bfloat16.
+ *   philox4x32_10         Random123 known-answer vectors.
+ *   normal/uniform fills  moments + distribution bounds (self-defined stream:
+ *                         "parity unpinned" with respect to the reference's
+ *                         cuRAND / oneMath streams, which nothing in the
+ *                         reference records).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+enum { OR_S8S8S32 = 0, OR_BF16BF16F32 = 1, OR_BF16BF16BF16 = 2, OR_F16F16F16 = 3 };
+enum { OR_ROW = 0, OR_COL = 1 };
+
+/* ------------------------------------------------------------------------ */
+/* 16-bit float conversions (round-to-nearest-even)                          */
+/* ------------------------------------------------------------------------ */
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+ORACLE_API float oracle_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+ORACLE_API uint16_t oracle_f32_to_bf16(float f) {
+  uint32_t u = f32_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+  uint32_t lsb = (u >> 16) & 1u;
+  u += 0x7fffu + lsb;
+  return (uint16_t)(u >> 16);
+}
+
+ORACLE_API float oracle_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  if (exp == 0) {
+    if (man == 0) return bits_f32(sign);
+    /* subnormal: value = man * 2^-24 */
+    float v = (float)man * 5.9604644775390625e-8f;
+    return bits_f32(f32_bits(v) | sign);
+  }
+  if (exp == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+  return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+ORACLE_API uint16_t oracle_f32_to_f16(float f) {
+  uint32_t u = f32_bits(f);
+  uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x3ffu)); /* NaN */
+  if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* >= 65520 rounds to inf */
+  if (a < 0x33000000u) {                                  /* < 2^-25 : rounds to 0   */
+    /* exactly 2^-25 ties to even (0); anything larger than 2^-25 goes up */
+    return sign;
+  }
+  int32_t e = (int32_t)(a >> 23) - 127;
+  uint32_t m = (a & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+  int shift;                                /* bits dropped from m */
+  uint32_t base;
+  if (e < -14) { /* subnormal half: unit is 2^-24 */
+    shift = 13 + (-14 - e);
+    base = 0;
+  } else {
+    shift = 13;
+    base = (uint32_t)(e + 15) << 10;
+    m &= 0x7fffffu;
+  }
+  uint32_t q = m >> shift;
+  uint32_t rem = m & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1u))) q++;
+  return (uint16_t)(sign | (base + q)); /* carry into exponent is intended */
+}
+
+static inline float round_to(int types, float v) {
+  if (types == OR_BF16BF16BF16) return oracle_bf16_to_f32(oracle_f32_to_bf16(v));
+  if (types == OR_F16F16F16) return oracle_f16_to_f32(oracle_f32_to_f16(v));
+  return v;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Literal loops (intel/utils/reference_kernel.hpp:16-28)                    */
+/* row-major A (m x k), row-major B (k x n), row-major C/D, C always read.   */
+/* ------------------------------------------------------------------------ */
+ORACLE_API void oracle_literal_s8s32(const int8_t* a, const int8_t* b, const int32_t* c, int32_t* d,
+                                     size_t m, size_t n, size_t k, int32_t alpha, int32_t beta) {
+  for (size_t gid = 0; gid < m * n; gid++) {
+    const size_t output_row = gid / n;
+    const size_t output_col = gid % n;
+    uint32_t acc = 0; /* two's-complement int32 arithmetic */
+    for (size_t i = 0; i < k; i++) {
+      acc += (uint32_t)((int32_t)a[output_row * k + i] * (int32_t)b[i * n + output_col]);
+    }
+    acc = (uint32_t)alpha * acc + (uint32_t)beta * (uint32_t)c[output_row * n + output_col];
+    d[output_row * n + output_col] = (int32_t)acc;
+  }
+}
+
+/* TOut = float instantiation; inputs already widened to float by the caller
+ * (the widening of bf16/fp16 to fp32 is exact).                              */
+ORACLE_API void oracle_literal_f32(const float* a, const float* b, const float* c, float* d,
+                                   size_t m, size_t n, size_t k, float alpha, float beta) {
+  for (size_t gid = 0; gid < m * n; gid++) {
+    const size_t output_row = gid / n;
+    const size_t output_col = gid % n;
+    float acc = 0.0f;
+    for (size_t i = 0; i < k; i++) {
+      acc += a[output_row * k + i] * b[i * n + output_col];
+    }
+    acc = alpha * acc + beta * c[output_row * n + output_col];
+    d[output_row * n + output_col] = acc;
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* General oracle: any layout, fp32 (or int32) sequential-k accumulate,      */
+/* generic_gemm epilogue (nvidia/kernels/generic_gemm.cuh:53-58).            */
+/* The j-inner loop order keeps each output's own summation order sequential */
+/* in k, exactly like the literal loop, while letting the compiler vectorise */
+/* across outputs.                                                           */
+/* ------------------------------------------------------------------------ */
+static size_t in_size(int types) { return types == OR_S8S8S32 ? 1 : 2; }
+static size_t out_size(int types) { return (types == OR_S8S8S32 || types == OR_BF16BF16F32) ? 4 : 2; }
+
+static float load_in_f32(int types, const void* p, size_t idx) {
+  const uint16_t* h = (const uint16_t*)p;
+  return types == OR_F16F16F16 ? oracle_f16_to_f32(h[idx]) : oracle_bf16_to_f32(h[idx]);
+}
+
+static float load_out_f32(int types, const void* p, size_t idx) {
+  if (types == OR_BF16BF16F32) return ((const float*)p)[idx];
+  if (types == OR_BF16BF16BF16) return oracle_bf16_to_f32(((const uint16_t*)p)[idx]);
+  return oracle_f16_to_f32(((const uint16_t*)p)[idx]);
+}
+
+static void store_out_f32(int types, void* p, size_t idx, float v) {
+  if (types == OR_BF16BF16F32) ((float*)p)[idx] = v;
+  else if (types == OR_BF16BF16BF16) ((uint16_t*)p)[idx] = oracle_f32_to_bf16(v);
+  else ((uint16_t*)p)[idx] = oracle_f32_to_f16(v);
+}
+
+/* Computes rows [row0, row1) of D.  Returns 0 on success. */
+ORACLE_API int oracle_gemm_rows(int types, const void* A, const void* B, const void* C, void* D,
+                                int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                                double alpha_d, double beta_d, int64_t row0, int64_t row1,
+                                int threads) {
+  if (types < 0 || types > 3 || M < 0 || N < 0 || K < 0) return 1;
+  if (row0 < 0 || row1 > M || row0 > row1) return 1;
+  if (M == 0 || N == 0) return 0;
+#ifdef _OPENMP
+  if (threads <= 0) threads = omp_get_max_threads();
+#else
+  threads = 1;
+#endif
+
+  if (types == OR_S8S8S32) {
+    const int8_t* a = (const int8_t*)A;
+    const int8_t* b = (const int8_t*)B;
+    const int32_t* c = (const int32_t*)C;
+    int32_t* d = (int32_t*)D;
+    const uint32_t alpha = (uint32_t)(int32_t)alpha_d, beta = (uint32_t)(int32_t)beta_d;
+    /* pure data movement: B as row-major K x N so the j loop is contiguous */
+    int8_t* bt = NULL;
+    if (layoutB == OR_COL && K > 0) {
+      bt = (int8_t*)malloc((size_t)K * N);
+      if (!bt) return 2;
+#pragma omp parallel for num_threads(threads) schedule(static)
+      for (int64_t p = 0; p < K; p++)
+        for (int64_t j = 0; j < N; j++) bt[p * N + j] = b[j * K + p];
+      b = bt;
+    }
+#pragma omp parallel num_threads(threads)
+    {
+      uint32_t* acc = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)N);
+#pragma omp for schedule(dynamic, 4)
+      for (int64_t i = row0; i < row1; i++) {
+        for (int64_t j = 0; j < N; j++) acc[j] = 0;
+        for (int64_t p = 0; p < K; p++) {
+          const int32_t av = layoutA == OR_ROW ? a[i * K + p] : a[p * M + i];
+          const int8_t* brow = b + p * N;
+          for (int64_t j = 0; j < N; j++) acc[j] += (uint32_t)(av * (int32_t)brow[j]);
+        }
+        for (int64_t j = 0; j < N; j++) {
+          uint32_t v = alpha * acc[j];
+          if (beta != 0) v += beta * (uint32_t)c[i * N + j];
+          d[i * N + j] = (int32_t)v;
+        }
+      }
+      free(acc);
+    }
+    free(bt);
+    return 0;
+  }
+
+  /* float paths */
+  const float alpha = round_to(types, (float)alpha_d);
+  const float beta = round_to(types, (float)beta_d);
+  float* bf = K > 0 ? (float*)malloc(sizeof(float) * (size_t)K * N) : NULL;
+  if (K > 0 && !bf) return 2;
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int64_t p = 0; p < K; p++)
+    for (int64_t j = 0; j < N; j++)
+      bf[p * N + j] = load_in_f32(types, B, layoutB == OR_ROW ? (size_t)(p * N + j) : (size_t)(j * K + p));
+
+#pragma omp parallel num_threads(threads)
+  {
+    float* acc = (float*)malloc(sizeof(float) * (size_t)N);
+#pragma omp for schedule(dynamic, 4)
+    for (int64_t i = row0; i < row1; i++) {
+      for (int64_t j = 0; j < N; j++) acc[j] = 0.0f;
+      for (int64_t p = 0; p < K; p++) {
+        const float av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
+        const float* brow = bf + p * N;
+        /* a*b is exact in fp32 for 16-bit inputs; one rounding per add */
+        for (int64_t j = 0; j < N; j++) acc[j] = acc[j] + av * brow[j];
+      }
+      for (int64_t j = 0; j < N; j++) {
+        /* generic_gemm.cuh:53-58, every operation rounded to TOut */
+        float val = round_to(types, acc[j]);
+        val = round_to(types, val * alpha);
+        if (beta != 0.0f) {
+          float bc = round_to(types, beta * load_out_f32(types, C, (size_t)(i * N + j)));
+          val = round_to(types, val + bc);
+        }
+        store_out_f32(types, D, (size_t)(i * N + j), val);
+      }
+    }
+    free(acc);
+  }
+  free(bf);
+  return 0;
+}
+
+ORACLE_API int oracle_gemm(int types, const void* A, const void* B, const void* C, void* D,
+                           int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                           double alpha, double beta, int threads) {
+  return oracle_gemm_rows(types, A, B, C, D, M, N, K, layoutA, layoutB, alpha, beta, 0, M, threads);
+}
+
+/* The literal one-work-item-per-output loop for any type pair and layout,
+ * parallelised as the reference parallelises it (one output element per
+ * work-item, reference_kernel.hpp:36-37 -> omp over the flattened index).
+ * Used as the CPU baseline timed beside the GPU number; accumulates in fp32
+ * (int32) and applies the same epilogue as oracle_gemm.                     */
+ORACLE_API int oracle_gemm_naive_rows(int types, const void* A, const void* B, const void* C, void* D,
+                                      int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                                      double alpha_d, double beta_d, int64_t row0, int64_t row1,
+                                      int threads) {
+  if (types < 0 || types > 3 || M < 0 || N < 0 || K < 0) return 1;
+  if (row0 < 0 || row1 > M || row0 > row1) return 1;
+  if (N == 0) return 0;
+#ifdef _OPENMP
+  if (threads <= 0) threads = omp_get_max_threads();
+#else
+  threads = 1;
+#endif
+  const float alpha = round_to(types, (float)alpha_d);
+  const float beta = round_to(types, (float)beta_d);
+  const uint32_t ialpha = (uint32_t)(int32_t)alpha_d, ibeta = (uint32_t)(int32_t)beta_d;
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int64_t gid = row0 * N; gid < row1 * N; gid++) {
+    const int64_t i = gid / N, j = gid % N;
+    if (types == OR_S8S8S32) {
+      const int8_t* a = (const int8_t*)A;
+      const int8_t* b = (const int8_t*)B;
+      uint32_t acc = 0;
+      for (int64_t p = 0; p < K; p++) {
+        int32_t av = layoutA == OR_ROW ? a[i * K + p] : a[p * M + i];
+        int32_t bv = layoutB == OR_ROW ? b[p * N + j] : b[j * K + p];
+        acc += (uint32_t)(av * bv);
+      }
+      uint32_t v = ialpha * acc;
+      if (ibeta != 0) v += ibeta * (uint32_t)((const int32_t*)C)[gid];
+      ((int32_t*)D)[gid] = (int32_t)v;
+    } else {
+      float acc = 0.0f;
+      for (int64_t p = 0; p < K; p++) {
+        float av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
+        float bv = load_in_f32(types, B, layoutB == OR_ROW ? (size_t)(p * N + j) : (size_t)(j * K + p));
+        acc = acc + av * bv;
+      }
+      float val = round_to(types, acc);
+      val = round_to(types, val * alpha);
+      if (beta != 0.0f) {
+        float bc = round_to(types, beta * load_out_f32(types, C, (size_t)gid));
+        val = round_to(types, val + bc);
+      }
+      store_out_f32(types, D, (size_t)gid, val);
+    }
+  }
+  return 0;
+}
+
+/* fp64-accumulated product (no epilogue rounding): truth for tolerance tests.
+ * out[i*N+j] = alpha * sum_p A(i,p) B(p,j) + beta * C(i,j), all in double.
+ * absout (optional) receives sum_p |A(i,p)| |B(p,j)| for error bounds.       */
+ORACLE_API int oracle_gemm_f64(int types, const void* A, const void* B, const void* C, double* out,
+                               double* absout, int64_t M, int64_t N, int64_t K, int layoutA,
+                               int layoutB, double alpha, double beta, int64_t row0, int64_t row1,
+                               int threads) {
+  if (types < 1 || types > 3) return 1;
+#ifdef _OPENMP
+  if (threads <= 0) threads = omp_get_max_threads();
+#else
+  threads = 1;
+#endif
+  double* bf = (double*)malloc(sizeof(double) * (size_t)(K > 0 ? K : 1) * N);
+  if (!bf) return 2;
+  for (int64_t p = 0; p < K; p++)
+    for (int64_t j = 0; j < N; j++)
+      bf[p * N + j] = load_in_f32(types, B, layoutB == OR_ROW ? (size_t)(p * N + j) : (size_t)(j * K + p));
+#pragma omp parallel num_threads(threads)
+  {
+    double* acc = (double*)malloc(sizeof(double) * (size_t)N * 2);
+    double* aac = acc + N;
+#pragma omp for schedule(dynamic, 4)
+    for (int64_t i = row0; i < row1; i++) {
+      for (int64_t j = 0; j < N; j++) acc[j] = 0.0, aac[j] = 0.0;
+      for (int64_t p = 0; p < K; p++) {
+        const double av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
+        const double* brow = bf + p * N;
+        for (int64_t j = 0; j < N; j++) {
+          acc[j] += av * brow[j];
+          aac[j] += fabs(av * brow[j]);
+        }
+      }
+      for (int64_t j = 0; j < N; j++) {
+        double v = alpha * acc[j];
+        if (beta != 0.0) v += beta * (double)load_out_f32(types, C, (size_t)(i * N + j));
+        out[(i - row0) * N + j] = v;
+        if (absout) absout[(i - row0) * N + j] = aac[j];
+      }
+    }
+    free(acc);
+  }
+  free(bf);
+  return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Philox4x32-10 (Salmon et al., SC'11), counter = element index, key = seed */
+/* ------------------------------------------------------------------------ */
+ORACLE_API void oracle_philox4x32_10(const uint32_t ctr_in[4], const uint32_t key_in[2], uint32_t out[4]) {
+  uint32_t c0 = ctr_in[0], c1 = ctr_in[1], c2 = ctr_in[2], c3 = ctr_in[3];
+  uint32_t k0 = key_in[0], k1 = key_in[1];
+  for (int r = 0; r < 10; r++) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+static inline void philox_elem(uint64_t seed, uint64_t idx, uint32_t out[4]) {
+  uint32_t ctr[4] = {(uint32_t)idx, (uint32_t)(idx >> 32), 0u, 0u};
+  uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  oracle_philox4x32_10(ctr, key, out);
+}
+
+/* --- transcendental-free-of-libm helpers: only IEEE-exact operations ------ *
+ * (+, *, /, sqrt, fma), so that any IEEE implementation that evaluates the  *
+ * same expression tree produces the same bits.                              */
+static inline float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+
+/* natural log of x in (0, 1]; |rel err| ~ 1e-7 */
+static float det_logf(float x) {
+  uint32_t u = f32_bits(x);
+  int32_t e = (int32_t)(u >> 23) - 127;
+  uint32_t mant = (u & 0x007fffffu) | 0x3f800000u; /* m in [1,2) */
+  float m = bits_f32(mant);
+  if (m > 1.41421356f) { m = m * 0.5f; e += 1; }   /* m in (0.707, 1.414] */
+  float s = (m - 1.0f) / (m + 1.0f);
+  float s2 = s * s;
+  float p = 0.0909090909f;            /* 1/11 */
+  p = fma_(p, s2, 0.1111111111f);     /* 1/9  */
+  p = fma_(p, s2, 0.1428571429f);     /* 1/7  */
+  p = fma_(p, s2, 0.2f);              /* 1/5  */
+  p = fma_(p, s2, 0.3333333333f);     /* 1/3  */
+  p = fma_(p, s2, 1.0f);
+  float lm = (s + s) * p;
+  return fma_((float)e, 0.693147180559945f, lm);
+}
+
+/* sin and cos of 2*pi*u for u in [0,1); |abs err| ~ 1e-7 */
+static void det_sincos2pi(float u, float* sn, float* cs) {
+  float t = u * 8.0f;                 /* exact */
+  int oct = (int)t;                   /* 0..7 */
+  float r = t - (float)oct;           /* exact, in [0,1) */
+  if (oct & 1) r = 1.0f - r;          /* reflect odd octants: exact */
+  float x = r * 0.785398163397448f;   /* angle in [0, pi/4] */
+  float x2 = x * x;
+  float sp = 2.7557319224e-6f;        /*  1/9! */
+  sp = fma_(sp, x2, -1.9841269841e-4f);
+  sp = fma_(sp, x2, 8.3333333333e-3f);
+  sp = fma_(sp, x2, -1.6666666667e-1f);
+  sp = fma_(sp, x2, 1.0f);
+  float s = x * sp;
+  float cp = 2.4801587302e-5f;        /*  1/8! */
+  cp = fma_(cp, x2, -1.3888888889e-3f);
+  cp = fma_(cp, x2, 4.1666666667e-2f);
+  cp = fma_(cp, x2, -0.5f);
+  cp = fma_(cp, x2, 1.0f);
+  float c = cp;
+  /* octant fix-up: angle = oct*pi/4 + (odd ? pi/4 - x : x) */
+  float so, co;
+  switch ((oct + 1) >> 1 & 3) {       /* nearest multiple of pi/2 */
+    case 0: so = s; co = c; break;
+    case 1: so = c; co = s; break;
+    case 2: so = s; co = c; break;
+    default: so = c; co = s; break;
+  }
+  /* signs by octant */
+  static const signed char ssign[8] = {1, 1, 1, 1, -1, -1, -1, -1};
+  static const signed char csign[8] = {1, 1, -1, -1, -1, -1, 1, 1};
+  *sn = ssign[oct] > 0 ? so : -so;
+  *cs = csign[oct] > 0 ? co : -co;
+}
+
+static inline float uniform01_open(uint32_t w) { /* (0,1]: (w>>8 + 1) * 2^-24, exact */
+  return (float)((w >> 8) + 1u) * 5.9604644775390625e-8f;
+}
+static inline float uniform01(uint32_t w) {      /* [0,1): (w>>8) * 2^-24, exact */
+  return (float)(w >> 8) * 5.9604644775390625e-8f;
+}
+
+ORACLE_API float oracle_normal_from_words(uint32_t w0, uint32_t w1) {
+  float u1 = uniform01_open(w0);
+  float u2 = uniform01(w1);
+  float rad = __builtin_sqrtf(-2.0f * det_logf(u1));
+  float sn, cs;
+  det_sincos2pi(u2, &sn, &cs);
+  (void)sn;
+  return rad * cs;
+}
+
+/* kind: 0 = int8 uniform [-128,127] (low byte of word 0)
+ *       1 = N(0,1)*scale      2 = U(-1,1)*scale      3 = integers {-1,0,1}
+ *           (kind 3 mirrors intel/test/utils.hpp:35-41: uniform(-2,2)
+ *            truncated toward zero, so every partial sum is exact)
+ * dtype: 0 = int8, 1 = bf16, 2 = fp16, 3 = fp32, 4 = int32                  */
+static float fill_value(int kind, float scale, uint64_t seed, uint64_t idx) {
+  uint32_t w[4];
+  philox_elem(seed, idx, w);
+  switch (kind) {
+    case 0: return (float)(int8_t)(w[0] & 0xffu);
+    case 1: return oracle_normal_from_words(w[0], w[1]) * scale;
+    case 2: return fma_(uniform01(w[0]), 2.0f, -1.0f) * scale;
+    default: return (float)(int32_t)fma_(uniform01(w[0]), 4.0f, -2.0f);
+  }
+}
+
+ORACLE_API int oracle_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t seed,
+                           int threads) {
+  if (count < 0 || dtype < 0 || dtype > 4 || kind < 0 || kind > 3) return 1;
+#ifdef _OPENMP
+  if (threads <= 0) threads = omp_get_max_threads();
+#else
+  threads = 1;
+#endif
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int64_t i = 0; i < count; i++) {
+    float v = fill_value(kind, scale, seed, (uint64_t)i);
+    switch (dtype) {
+      case 0: ((int8_t*)dst)[i] = (int8_t)v; break;
+      case 1: ((uint16_t*)dst)[i] = oracle_f32_to_bf16(v); break;
+      case 2: ((uint16_t*)dst)[i] = oracle_f32_to_f16(v); break;
+      case 3: ((float*)dst)[i] = v; break;
+      default: ((int32_t*)dst)[i] = (int32_t)v; break;
+    }
+  }
+  return 0;
+}
+
+ORACLE_API int oracle_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+ORACLE_API size_t oracle_in_size(int types) { return in_size(types); }
+ORACLE_API size_t oracle_out_size(int types) { return out_size(types); }
