@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Headline benchmark: bf16 x bf16 -> f32 GEMM, M=N=K=4096, A row-major, B column-major, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu-baseline]
+
+One "step" is one launch of the GEMM on one of P rotating input sets that are already
+resident in HBM (P is sized so that the 256 MB Infinity Cache cannot hold the operands
+between launches).  Prints ONE JSON line.  `value` is 2*M*N*K*steps / wall time of the
+timed region; `roofline.achieved` uses the mean HIP-event duration of the same launches.
+Beside it the line carries the int8 8192^3 and the skinny (decode) shapes, the hipBLASLt
+comparator when its library is built, and the CPU restatement of the reference GEMM timed
+on this machine's host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0}  # dense MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+INFINITY_CACHE_BYTES = 256 * 1000 * 1000
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extras", action="store_true", help="skip the s8 8192^3 and skinny side measurements")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures ONE GPU (the GEMM path has no cross-GPU exchange; "
+              "shard N or M across GPUs and run the same kernel per shard). Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    capi = importlib.import_module("gemm-zoo_amd.capi")  # raises if the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream()
+    sptr = stream.cuda_stream
+
+    IN_T = {capi.S8S8S32: torch.int8, capi.BF16BF16F32: torch.bfloat16, capi.BF16BF16BF16: torch.bfloat16,
+            capi.F16F16F16: torch.float16}
+    OUT_T = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
+             capi.F16F16F16: torch.float16}
+    IN_DT = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
+             capi.F16F16F16: capi.DT_F16}
+
+    def make_sets(types, m, n, k, scale_b=1.0, seed0=2025):
+        """P rotating (A, B) sets + one D, filled on the device (seeds 2025, 2026, ... as the reference harness)."""
+        es = capi.IN_SIZE[types]
+        problem_bytes = es * (m * k + k * n) + capi.OUT_SIZE[types] * m * n
+        p = INFINITY_CACHE_BYTES // problem_bytes + 1
+        kind = capi.FILL_INT8_UNIFORM if types == capi.S8S8S32 else capi.FILL_NORMAL
+        sets = []
+        for j in range(p):
+            a = torch.empty(m * k, dtype=IN_T[types], device=dev)
+            b = torch.empty(k * n, dtype=IN_T[types], device=dev)
+            capi.fill(a, m * k, IN_DT[types], kind, 1.0, seed0 + 3 * j, sptr)
+            capi.fill(b, k * n, IN_DT[types], kind, scale_b, seed0 + 3 * j + 1, sptr)
+            sets.append((a, b))
+        d = torch.empty(m * n, dtype=OUT_T[types], device=dev)
+        return sets, d, problem_bytes
+
+    def timed(types, m, n, k, la, lb, steps, warmup, rung=capi.RUNG_AUTO, variant=0, scale_b=1.0, verify=True):
+        sets, d, problem_bytes = make_sets(types, m, n, k, scale_b)
+        p = len(sets)
+
+        def launch(i):
+            a, b = sets[i % p]
+            capi.gemm(types, a, b, None, d, m, n, k, la, lb, 1, 0, rung, variant, sptr)
+
+        if verify:  # verify-once, against an independent rung of the ladder (sequential-k LDS kernel)
+            launch(0)
+            ref = torch.empty_like(d)
+            a, b = sets[0]
+            capi.gemm(types, a, b, None, ref, m, n, k, la, lb, 1, 0, capi.RUNG_LDS_TILED, 0, sptr)
+            if types == capi.S8S8S32:
+                ndiff = capi.compare(d, ref, m * n, capi.DT_INT32, 0.0, sptr)
+            else:
+                dt = {capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16, capi.F16F16F16: capi.DT_F16}[types]
+                # sanity bound only (parity proper lives in tests/): fp32 accumulation in a different order, so allow
+                # 1e-3 of the output scale for fp32 out and one 16-bit ulp at 4 sigma for 16-bit out
+                scale = float(torch.sqrt(torch.tensor(float(k)))) * scale_b
+                tol = (1e-3 if types == capi.BF16BF16F32 else 4e-2) * scale
+                ndiff = capi.compare(d, ref, m * n, dt, tol, sptr)
+            if ndiff:
+                raise RuntimeError(f"verification failed: {ndiff} elements differ ({capi.TYPES_NAMES[types]} {m}x{n}x{k})")
+            del ref
+        for i in range(warmup):
+            launch(i)
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            starts[i].record(stream)
+            launch(i + 1)
+            stops[i].record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ev = sorted(s.elapsed_time(e) for s, e in zip(starts, stops))
+        wall_ms = (t1 - t0) * 1e3 / steps
+        return {"wall_ms": wall_ms, "kernel_ms_mean": sum(ev) / len(ev), "kernel_ms_median": ev[len(ev) // 2],
+                "problem_bytes": problem_bytes, "sets": p}
+
+    # ---------------- headline: bf16 4096^3, A row-major, B column-major, f32 out ----------------
+    M = N = K = 4096
+    flops = 2.0 * M * N * K
+    r = timed(capi.BF16BF16F32, M, N, K, capi.ROW_MAJOR, capi.COL_MAJOR, args.steps, args.warmup)
+    plan = capi.plan(capi.BF16BF16F32, M, N, K, capi.ROW_MAJOR, capi.COL_MAJOR).as_dict()
+    value = flops / (r["wall_ms"] * 1e-3) / 1e12
+    achieved = flops / (r["kernel_ms_mean"] * 1e-3) / 1e12
+
+    out = {
+        "metric": "TFLOPS/TOPS at bf16 4096^3 and s8 8192^3; % of MFMA peak; GB/s skinny M",
+        "value": round(value, 2),
+        "unit": "TFLOPS (bf16 4096^3)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "bf16 x bf16 -> f32 GEMM M=N=K=4096, A row-major, B column-major, N(0,1) inputs, "
+                               "alpha=1 beta=0, fp32 accumulate",
+                   "rotating_input_sets": r["sets"], "plan": plan},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": None,
+                     "kernel_ms_mean": round(r["kernel_ms_mean"], 5), "kernel_ms_median": round(r["kernel_ms_median"], 5)},
+    }
+
+    # ---------------- side measurements named by the metric ----------------
+    if not args.no_extras:
+        extras = {}
+        m8 = 8192
+        r8 = timed(capi.S8S8S32, m8, m8, m8, capi.ROW_MAJOR, capi.COL_MAJOR, 10, 2)
+        tops = 2.0 * m8 ** 3 / (r8["kernel_ms_mean"] * 1e-3) / 1e12
+        extras["s8_8192"] = {"tops": round(tops, 2), "frac_of_int8_peak": round(tops / PEAK_TFLOPS["s8"], 4),
+                             "kernel_ms_mean": round(r8["kernel_ms_mean"], 5)}
+        sk = {}
+        for m in (1, 8, 32, 128):
+            rs = timed(capi.BF16BF16BF16, m, 14336, 4096, capi.ROW_MAJOR, capi.COL_MAJOR, 30, 5, scale_b=0.02)
+            gbs = rs["problem_bytes"] / (rs["kernel_ms_mean"] * 1e-3) / 1e9
+            sk[f"M={m}"] = {"gb_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                            "kernel_us_mean": round(rs["kernel_ms_mean"] * 1e3, 2)}
+        extras["skinny_bf16_N14336_K4096"] = sk
+        out["extras"] = extras
+
+    # ---------------- CPU restatement of the reference GEMM on this box's host cores ----------------
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(M, N, K, args.cpu_seconds)
+
+    print(json.dumps(out))
+    return 0
+
+
+def cpu_baseline(M, N, K, target_seconds):
+    """The oracle's literal one-output-per-work-item loop on a band of rows of the same workload."""
+    sys.path.insert(0, str(ROOT / "tests"))
+    import oracle_lib as O
+
+    threads = int(O.lib.oracle_num_threads())
+    a = O.fill(M * K, O.DT_BF16, O.FILL_NORMAL, 1.0, 2025)
+    b = O.fill(K * N, O.DT_BF16, O.FILL_NORMAL, 1.0, 2026)
+    # calibrate on a few rows, then size the band for about target_seconds
+    r0 = max(threads // 4, 2)
+    t = time.perf_counter()
+    O.gemm(O.BF16BF16F32, a, b, None, M, N, K, O.ROW, O.COL, 1.0, 0.0, threads=threads, rows=(0, r0), naive=True)
+    dt = time.perf_counter() - t
+    rows = int(min(M, max(r0, target_seconds / max(dt / r0, 1e-9))))
+    t = time.perf_counter()
+    O.gemm(O.BF16BF16F32, a, b, None, M, N, K, O.ROW, O.COL, 1.0, 0.0, threads=threads, rows=(0, rows), naive=True)
+    dt = time.perf_counter() - t
+    tflops = 2.0 * rows * N * K / dt / 1e12
+    return {"value": round(tflops, 6), "unit": "TFLOPS (bf16 4096^3)", "cores": threads, "kind": "port",
+            "sample": f"rows [0,{rows}) of {M} of the same bf16 4096^3 problem ({rows}x{N}x{K} MACs, {dt:.1f} s), "
+                      f"literal one-output-per-work-item loop with fp32 accumulate, OpenMP over outputs; "
+                      f"full problem would take {dt * M / rows:.0f} s"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -21,7 +21,8 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 # packed fp32 VALU instructions are switched off for every translation unit
 COMMON = [
-    "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
+    "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     "-Wno-option-ignored", "-Wno-unused-function",
@@ -29,7 +30,8 @@ COMMON = [
 
 PRODUCT_SOURCES = [
     "gz_api.hip", "gz_fill_compare.hip", "rung0_naive.hip", "rung1_coalesced.hip",
-    "rung23_lds.hip", "rung4_mfma.hip", "rung5_skinny.hip",
+    "rung23_lds.hip", "rung4_mfma_s8s8s32.hip", "rung4_mfma_bf16bf16f32.hip", "rung4_mfma_bf16bf16bf16.hip",
+    "rung4_mfma_f16f16f16.hip", "rung5_skinny.hip",
 ]
 COMPARATOR_SOURCES = ["gz_hipblaslt.cpp"]
 

@@ -89,7 +89,12 @@ static int run(const void* A, const void* B, const void* C, void* D, int64_t M, 
   g.alpha = alpha; g.beta = beta;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
-  switch (resolve_rung(TYPES, M, N, K, layoutA, layoutB, rung)) {
+  int resolved = resolve_rung(TYPES, M, N, K, layoutA, layoutB, rung);
+  // the streaming kernel needs 16-byte aligned operands; AUTO falls back to the tiled kernel otherwise
+  if (rung == GZ_RUNG_AUTO && resolved == GZ_RUNG_SKINNY &&
+      ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15u))
+    resolved = GZ_RUNG_MFMA;
+  switch (resolved) {
     case GZ_RUNG_NAIVE: return launch_naive<TYPES>(g, variant, s);
     case GZ_RUNG_COALESCED: return launch_coalesced<TYPES>(g, variant, s);
     case GZ_RUNG_LDS_TILED: return launch_lds_tiled<TYPES>(g, variant, s);

@@ -1,6 +1,12 @@
 // Shared device/host definitions for the gfx950 GEMM ladder.
 #pragma once
 
+// Every translation unit of the library is built with -ffp-contract=off and repeats it here:
+// a*b+c written as two operations must round twice, so that the epilogue and the seeded fill
+// produce the same bits as a host evaluation of the same expression.  Fused multiply-adds are
+// always spelled __builtin_fmaf.
+#pragma clang fp contract(off)
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -88,8 +94,8 @@ template <int TYPES> __host__ __device__ inline float round_out(float v) {
 
 // Explicit single-rounding fp32 operations: the epilogue must not be fused into
 // an FMA, so that its value is the same on every rung.
-__device__ inline float mul_rn(float a, float b) { return __fmul_rn(a, b); }
-__device__ inline float add_rn(float a, float b) { return __fadd_rn(a, b); }
+__device__ inline float mul_rn(float a, float b) { return a * b; }
+__device__ inline float add_rn(float a, float b) { return a + b; }
 
 // Epilogue shared by every rung.  `c_ptr` is dereferenced only when beta != 0.
 template <int TYPES>

@@ -13,8 +13,6 @@
 // threshold) and test::compare_results (intel/test/utils.hpp:47-73, exact).
 #include "gz_common.hpp"
 
-#pragma clang fp contract(off)
-
 namespace gz {
 
 __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
@@ -32,39 +30,43 @@ __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint
 }
 
 __device__ inline float fma_rn(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+// plain IEEE operations (contraction is off; fp32 divide and square root are correctly rounded by default)
+__device__ inline float sub_rn(float a, float b) { return a - b; }
+__device__ inline float div_rn(float a, float b) { return a / b; }
+__device__ inline float sqrt_rn(float a) { return __builtin_sqrtf(a); }
 
 // natural log on (0, 1]: exponent split + atanh series, IEEE-exact primitives only
 __device__ inline float det_logf(float x) {
   const uint32_t u = __builtin_bit_cast(uint32_t, x);
   int e = (int)(u >> 23) - 127;
   float m = __builtin_bit_cast(float, (u & 0x007fffffu) | 0x3f800000u);
-  if (m > 1.41421356f) { m = __fmul_rn(m, 0.5f); e += 1; }
-  const float s = __fdiv_rn(__fsub_rn(m, 1.0f), __fadd_rn(m, 1.0f));
-  const float s2 = __fmul_rn(s, s);
+  if (m > 1.41421356f) { m = mul_rn(m, 0.5f); e += 1; }
+  const float s = div_rn(sub_rn(m, 1.0f), add_rn(m, 1.0f));
+  const float s2 = mul_rn(s, s);
   float p = 0.0909090909f;
   p = fma_rn(p, s2, 0.1111111111f);
   p = fma_rn(p, s2, 0.1428571429f);
   p = fma_rn(p, s2, 0.2f);
   p = fma_rn(p, s2, 0.3333333333f);
   p = fma_rn(p, s2, 1.0f);
-  const float lm = __fmul_rn(__fadd_rn(s, s), p);
+  const float lm = mul_rn(add_rn(s, s), p);
   return fma_rn((float)e, 0.693147180559945f, lm);
 }
 
 // cos(2 pi u), u in [0,1): octant reduction is exact, then a Taylor polynomial on [0, pi/4]
 __device__ inline float det_cos2pi(float u) {
-  const float t = __fmul_rn(u, 8.0f);
+  const float t = mul_rn(u, 8.0f);
   const int oct = (int)t;
-  float r = __fsub_rn(t, (float)oct);
-  if (oct & 1) r = __fsub_rn(1.0f, r);
-  const float x = __fmul_rn(r, 0.785398163397448f);
-  const float x2 = __fmul_rn(x, x);
+  float r = sub_rn(t, (float)oct);
+  if (oct & 1) r = sub_rn(1.0f, r);
+  const float x = mul_rn(r, 0.785398163397448f);
+  const float x2 = mul_rn(x, x);
   float sp = 2.7557319224e-6f;
   sp = fma_rn(sp, x2, -1.9841269841e-4f);
   sp = fma_rn(sp, x2, 8.3333333333e-3f);
   sp = fma_rn(sp, x2, -1.6666666667e-1f);
   sp = fma_rn(sp, x2, 1.0f);
-  const float s = __fmul_rn(x, sp);
+  const float s = mul_rn(x, sp);
   float cp = 2.4801587302e-5f;
   cp = fma_rn(cp, x2, -1.3888888889e-3f);
   cp = fma_rn(cp, x2, 4.1666666667e-2f);
@@ -77,9 +79,9 @@ __device__ inline float det_cos2pi(float u) {
   return neg ? -mag : mag;
 }
 
-__device__ inline float uniform01(uint32_t w) { return __fmul_rn((float)(w >> 8), 5.9604644775390625e-8f); }
+__device__ inline float uniform01(uint32_t w) { return mul_rn((float)(w >> 8), 5.9604644775390625e-8f); }
 __device__ inline float uniform01_open(uint32_t w) {
-  return __fmul_rn((float)((w >> 8) + 1u), 5.9604644775390625e-8f);
+  return mul_rn((float)((w >> 8) + 1u), 5.9604644775390625e-8f);
 }
 
 __device__ inline float fill_value(int kind, float scale, uint64_t seed, uint64_t idx) {
@@ -88,10 +90,10 @@ __device__ inline float fill_value(int kind, float scale, uint64_t seed, uint64_
   switch (kind) {
     case 0: return (float)(int8_t)(w[0] & 0xffu);
     case 1: {
-      const float rad = __fsqrt_rn(__fmul_rn(-2.0f, det_logf(uniform01_open(w[0]))));
-      return __fmul_rn(__fmul_rn(rad, det_cos2pi(uniform01(w[1]))), scale);
+      const float rad = sqrt_rn(mul_rn(-2.0f, det_logf(uniform01_open(w[0]))));
+      return mul_rn(mul_rn(rad, det_cos2pi(uniform01(w[1]))), scale);
     }
-    case 2: return __fmul_rn(fma_rn(uniform01(w[0]), 2.0f, -1.0f), scale);
+    case 2: return mul_rn(fma_rn(uniform01(w[0]), 2.0f, -1.0f), scale);
     default: return (float)(int32_t)fma_rn(uniform01(w[0]), 4.0f, -2.0f);
   }
 }

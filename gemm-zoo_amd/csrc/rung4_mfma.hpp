@@ -16,6 +16,7 @@
 //
 // Stands in for nvidia/kernels/sm_80/{bf16,fp16}_mma_gemm.cuh and
 // intel/kernels/xe_gemm_*_m8k16.hpp (same operation, new design).
+#pragma once
 #include "gz_common.hpp"
 #include "gz_mfma_cfg.hpp"
 
@@ -349,10 +350,5 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipS
   set_error("mfma rung: variant %d not built", cfg.id);
   return GZ_ERR_UNSUPPORTED;
 }
-
-template int launch_mfma<GZ_S8S8S32>(const GemmArgs<GZ_S8S8S32>&, int, hipStream_t);
-template int launch_mfma<GZ_BF16BF16F32>(const GemmArgs<GZ_BF16BF16F32>&, int, hipStream_t);
-template int launch_mfma<GZ_BF16BF16BF16>(const GemmArgs<GZ_BF16BF16BF16>&, int, hipStream_t);
-template int launch_mfma<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hipStream_t);
 
 }  // namespace gz

@@ -1,0 +1,114 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports what the header
+declares, validates arguments before touching the device, and plans launches sensibly."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def declared_symbols():
+    text = (ROOT / "include" / "gemm_zoo.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gz_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(capi):
+    names = declared_symbols()
+    assert len(names) >= 13 and set(names) == set(capi.EXPORTS)
+    raw = ctypes.CDLL(str(capi.LIB_PATH))
+    for n in names:
+        assert hasattr(raw, n), n
+
+
+def test_version_and_names(capi):
+    assert capi.lib.gz_version() >= 1
+    assert [capi.rung_name(r) for r in range(capi.NUM_RUNGS)] == [
+        "naive", "coalesced", "lds_tiled", "double_buffered", "mfma", "skinny"]
+    assert capi.lib.gz_types_name(capi.S8S8S32) == b"s8s8s32"
+    assert capi.variant_count(capi.BF16BF16F32, capi.RUNG_MFMA) >= 3
+    assert capi.variant_count(capi.S8S8S32, capi.RUNG_SKINNY) == 0
+
+
+@pytest.mark.parametrize("kwargs,status", [
+    (dict(types=9), 1), (dict(m=-1), 1), (dict(k=-5), 1), (dict(layout_a=2), 1), (dict(layout_b=-1), 1),
+    (dict(rung=6), 1), (dict(rung=-2), 1), (dict(variant=-1), 1),
+    (dict(m=1 << 20, k=1 << 20), 2),            # 2^40 elements
+    (dict(rung=4, variant=99), 2),
+    (dict(rung=0, variant=1), 2),
+    (dict(types=0, rung=5), 2),                 # no int8 streaming kernel
+    (dict(rung=5, m=64, layout_b=1), 2),        # M too large for the streaming kernel
+    (dict(rung=5, m=8, layout_b=0), 2),         # needs column-major weights
+    (dict(rung=5, m=8, layout_b=1, k=100), 2),  # K not a whole number of super-steps
+])
+def test_plan_rejects_bad_requests(capi, kwargs, status):
+    args = dict(types=1, m=128, n=128, k=128, layout_a=0, layout_b=0, rung=-1, variant=0)
+    args.update(kwargs)
+    with pytest.raises(capi.GzError) as e:
+        capi.plan(**args)
+    assert e.value.status == status and str(e.value)
+
+
+def test_gemm_entry_points_validate_before_any_device_work(capi):
+    """Bad arguments must come back as status codes without a GPU being present."""
+    for types in range(4):
+        with pytest.raises(capi.GzError) as e:
+            capi.gemm(types, 0, 0, 0, 0, 16, 16, 16)  # NULL operands
+        assert e.value.status == capi.ERR_BAD_ARG
+        with pytest.raises(capi.GzError) as e:
+            capi.gemm(types, 64, 64, 0, 64, 16, 16, 16, beta=1)  # beta != 0 needs C
+        assert e.value.status == capi.ERR_BAD_ARG and "C is NULL" in str(e.value)
+        with pytest.raises(capi.GzError) as e:
+            capi.gemm(types, 64, 64, 64, 64, -1, 16, 16)
+        assert e.value.status == capi.ERR_BAD_ARG
+        with pytest.raises(capi.GzError) as e:
+            capi.gemm(types, 64, 64, 64, 64, 16, 16, 16, layout_a=7)
+        assert e.value.status == capi.ERR_BAD_ARG
+        # empty outputs are a no-op, whatever the pointers
+        capi.gemm(types, 0, 0, 0, 0, 0, 16, 16)
+        capi.gemm(types, 0, 0, 0, 0, 16, 0, 16)
+    st = capi.lib.gz_gemm(0, 64, 64, 64, 64, 4, 4, 4, 0, 0, 1.5, 0.0, -1, 0, None)
+    assert st == capi.ERR_BAD_ARG and "integral" in capi.last_error()
+    assert capi.lib.gz_gemm(17, 64, 64, 64, 64, 4, 4, 4, 0, 0, 1.0, 0.0, -1, 0, None) == capi.ERR_BAD_ARG
+    assert capi.lib.gz_fill(None, 10, 0, 0, 1.0, 1, None) == capi.ERR_BAD_ARG
+    assert capi.lib.gz_fill(None, 0, 0, 0, 1.0, 1, None) == capi.OK
+    assert capi.lib.gz_fill(64, 10, 9, 0, 1.0, 1, None) == capi.ERR_BAD_ARG
+    assert capi.lib.gz_compare(None, None, 10, 0, 0.0, None, None) == capi.ERR_BAD_ARG
+    assert capi.lib.gz_compare(None, None, 0, 0, 0.0, None, None) == capi.OK
+
+
+def test_plan_headline_configs(capi):
+    # bf16 4096^3: 256 tiles of 256x256 = one per compute unit
+    p = capi.plan(capi.BF16BF16F32, 4096, 4096, 4096, 0, 1)
+    assert (p.rung, p.tile_m, p.tile_n, p.tile_k, p.grid) == (capi.RUNG_MFMA, 256, 256, 64, 256)
+    assert p.lds_bytes <= 160 * 1024 and p.vector_bytes_a == 16 and p.vector_bytes_b == 16
+    # int8 consumes 128 k per slab
+    p = capi.plan(capi.S8S8S32, 8192, 8192, 8192, 0, 1)
+    assert (p.rung, p.tile_k, p.grid) == (capi.RUNG_MFMA, 128, 1024)
+    # ragged fp16 problem: ceil-div grid, only 2-byte aligned lines
+    p = capi.plan(capi.F16F16F16, 4095, 4097, 1023, 0, 0)
+    assert p.grid == -(-4095 // p.tile_m) * -(-4097 // p.tile_n)
+    assert p.vector_bytes_a == 2 and p.vector_bytes_b == 2
+    # decode shapes go to the streaming kernel under AUTO, big M does not
+    for m in (1, 8, 32):
+        p = capi.plan(capi.BF16BF16BF16, m, 14336, 4096, 0, 1)
+        assert p.rung == capi.RUNG_SKINNY and p.grid * p.tile_n >= 14336 and p.tile_m >= m
+    assert capi.plan(capi.BF16BF16BF16, 128, 14336, 4096, 0, 1).rung == capi.RUNG_MFMA
+    # a small problem shrinks the tile so that more work-groups exist
+    small = capi.plan(capi.BF16BF16F32, 1024, 1024, 1024, 0, 1)
+    assert small.tile_m * small.tile_n < 256 * 256
+    # an explicit variant is honoured; a device with little LDS refuses the big tile
+    assert capi.plan(capi.BF16BF16F32, 1024, 1024, 1024, 0, 1, capi.RUNG_MFMA, 1).tile_m == 256
+    with pytest.raises(capi.GzError) as e:
+        capi.plan(capi.BF16BF16F32, 4096, 4096, 4096, 0, 1, capi.RUNG_MFMA, 1, num_cus=256, lds_per_cu=64 * 1024)
+    assert e.value.status == capi.ERR_UNSUPPORTED
+
+
+def test_plan_every_rung_and_type(capi):
+    for types in range(4):
+        for rung in range(5):
+            p = capi.plan(types, 300, 500, 700, 0, 0, rung)
+            assert p.rung == rung and p.grid >= 1 and p.threads in (128, 256, 512, 1024)
+            assert p.grid * p.tile_m * p.tile_n >= 300 * 500

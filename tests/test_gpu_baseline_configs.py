@@ -1,0 +1,125 @@
+"""The five BASELINE configurations at their full sizes, through the C ABI.
+
+Small ones are compared element for element with the CPU oracle.  The large ones (4096^3, 8192^3)
+are checked through size-independent properties that are exact for integers -- D x = A (B x) and
+x^T D = (x^T A) B in int64 for random x -- plus bands of rows against the oracle.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    return gpu_util
+
+
+def device_inputs(G, types, m, n, k, kind, seed, scale_b=1.0):
+    it = torch.int8 if types == O.S8S8S32 else torch.int16
+    a = torch.empty(m * k, dtype=it, device="cuda"); b = torch.empty(k * n, dtype=it, device="cuda")
+    G.capi.fill(a, m * k, O.IN_DT[types], kind, 1.0, seed); G.capi.fill(b, k * n, O.IN_DT[types], kind, scale_b, seed + 1)
+    torch.cuda.synchronize()
+    ha = a.cpu().numpy(); hb = b.cpu().numpy()
+    if types != O.S8S8S32:
+        ha = ha.view(np.uint16); hb = hb.view(np.uint16)
+    return a, b, ha, hb
+
+
+def test_c1_s8_1024_row_row_bit_exact_every_rung(G):
+    m = n = k = 1024
+    a, b, c = O.make_inputs(O.S8S8S32, m, n, k, seed=2025)
+    ref = O.gemm(O.S8S8S32, a, b, None, m, n, k, O.ROW, O.ROW, 1, 0)
+    lit = np.zeros((m, n), np.int32)  # the literal reference loop on a band, as a cross-check of the checker
+    band = O.gemm(O.S8S8S32, a, b, None, m, n, k, O.ROW, O.ROW, 1, 0, rows=(100, 116), naive=True)
+    assert np.array_equal(band[100:116], ref[100:116])
+    for rung in (-1, 0, 1, 2, 3, 4):
+        got = G.run_gemm(O.S8S8S32, a, b, None, m, n, k, O.ROW, O.ROW, 1, 0, rung)
+        assert np.array_equal(got, ref), rung
+    ref11 = O.gemm(O.S8S8S32, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1)
+    assert np.array_equal(G.run_gemm(O.S8S8S32, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1, -1), ref11)
+
+
+def test_c2_bf16_4096_row_col_f32(G):
+    m = n = k = 4096
+    types = O.BF16BF16F32
+    a, b, ha, hb = device_inputs(G, types, m, n, k, O.FILL_NORMAL, 2025)
+    assert np.array_equal(ha, O.fill(m * k, O.DT_BF16, O.FILL_NORMAL, 1.0, 2025))  # same bytes on both sides
+    d = torch.empty(m * n, dtype=torch.float32, device="cuda")
+    G.capi.gemm(types, a, b, None, d, m, n, k, O.ROW, O.COL, 1, 0)
+    torch.cuda.synchronize()
+    got = d.cpu().numpy().reshape(m, n)
+    for r0 in (0, 1777, 4088):  # bands of rows against fp64 truth and against the sequential fp32 oracle
+        truth, _ = O.gemm_f64(types, ha, hb, None, m, n, k, O.ROW, O.COL, 1, 0, rows=(r0, r0 + 8))
+        G.assert_within(types, got[r0:r0 + 8], truth, f"C2 rows {r0}")
+        ref = O.gemm(types, ha, hb, None, m, n, k, O.ROW, O.COL, 1, 0, rows=(r0, r0 + 8))[r0:r0 + 8]
+        G.assert_within(types, got[r0:r0 + 8], ref.astype(np.float64), f"C2 rows {r0} vs fp32 oracle")
+    # Freivalds: D x == A (B x) in fp64, for every row at once
+    rng = np.random.default_rng(0)
+    x = rng.choice([-1.0, 1.0], n)
+    A = O.bf16_to_f32(ha).reshape(m, k).astype(np.float64); Bt = O.bf16_to_f32(hb).reshape(n, k).astype(np.float64)
+    lhs = got.astype(np.float64) @ x
+    rhs = A @ (x @ Bt)
+    scale = np.sqrt(k * n)  # magnitude of a row's signed sum
+    assert np.abs(lhs - rhs).max() <= 1e-4 * scale
+    # integer-valued inputs: bit-exact at full size
+    G.capi.fill(a, m * k, O.DT_BF16, O.FILL_SMALL_INT, 1.0, 7); G.capi.fill(b, k * n, O.DT_BF16, O.FILL_SMALL_INT, 1.0, 8)
+    G.capi.gemm(types, a, b, None, d, m, n, k, O.ROW, O.COL, 1, 0)
+    torch.cuda.synchronize()
+    A = O.bf16_to_f32(a.cpu().numpy().view(np.uint16)).reshape(m, k); Bt = O.bf16_to_f32(b.cpu().numpy().view(np.uint16)).reshape(n, k)
+    want = (A.astype(np.float64) @ Bt.T.astype(np.float64))
+    assert np.array_equal(d.cpu().numpy().reshape(m, n).astype(np.float64), want)
+
+
+def test_c3_s8_8192_row_col_bit_exact(G):
+    m = n = k = 8192
+    types = O.S8S8S32
+    a, b, ha, hb = device_inputs(G, types, m, n, k, O.FILL_INT8_UNIFORM, 2025)
+    d = torch.empty(m * n, dtype=torch.int32, device="cuda")
+    G.capi.gemm(types, a, b, None, d, m, n, k, O.ROW, O.COL, 1, 0)
+    torch.cuda.synchronize()
+    got = d.cpu().numpy().reshape(m, n)
+    A = ha.reshape(m, k).astype(np.int64); Bt = hb.reshape(n, k).astype(np.int64)
+    rng = np.random.default_rng(1)
+    for _ in range(2):  # exact in int64: |entries| <= 2^27 * 8192 * 3
+        x = rng.integers(-3, 4, n).astype(np.int64)
+        assert np.array_equal(got.astype(np.int64) @ x, A @ (Bt.T @ x) if False else A @ (x @ Bt))
+        y = rng.integers(-3, 4, m).astype(np.int64)
+        assert np.array_equal(y @ got.astype(np.int64), (y @ A) @ Bt.T)
+    for r0 in (0, 4093, 8184):
+        ref = O.gemm(types, ha, hb, None, m, n, k, O.ROW, O.COL, 1, 0, rows=(r0, r0 + 8))
+        assert np.array_equal(got[r0:r0 + 8], ref[r0:r0 + 8])
+
+
+def test_c4_f16_ragged_row_row(G):
+    m, n, k = 4095, 4097, 1023
+    types = O.F16F16F16
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_UNIFORM_PM1, seed=2025)
+    got = G.run_gemm(types, a, b, None, m, n, k, O.ROW, O.ROW, 1, 0, -1)
+    ref = O.gemm(types, a, b, None, m, n, k, O.ROW, O.ROW, 1, 0)
+    G.assert_within(types, got, O.out_to_f64(types, ref), "C4 vs oracle")
+    truth, _ = O.gemm_f64(types, a, b, None, m, n, k, O.ROW, O.ROW, 1, 0, rows=(4000, 4095))
+    G.assert_within(types, got[4000:], truth, "C4 last rows vs fp64 truth")
+    # exact on integer-valued inputs, with beta
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=3)
+    got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1, -1)
+    assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1))
+
+
+@pytest.mark.parametrize("m", [1, 8, 32, 128])
+def test_c5_skinny_bf16(G, m):
+    n, k = 14336, 4096
+    types = O.BF16BF16BF16
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_NORMAL, seed=2025, scale_b=0.02)
+    got = G.run_gemm(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0, -1)
+    truth, _ = O.gemm_f64(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0)
+    G.assert_within(types, got, truth, f"C5 M={m} vs fp64 truth")
+    ref = O.gemm(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0)
+    G.assert_within(types, got, O.out_to_f64(types, ref), f"C5 M={m} vs oracle")
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=4)
+    got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1, -1)
+    assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1))

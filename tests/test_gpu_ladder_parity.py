@@ -1,0 +1,148 @@
+"""GPU parity of every rung, type bundle and layout against the CPU oracle, through the C ABI."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+LAYOUTS = list(itertools.product((O.ROW, O.COL), repeat=2))
+ALL_TYPES = (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16)
+VALU_RUNGS = (0, 1, 2, 3)
+MFMA = 4
+SKINNY = 5
+# ragged, tiny, tile-multiple and "one past a tile" shapes
+SHAPES = [(1, 1, 1), (3, 5, 7), (64, 64, 64), (65, 63, 33), (100, 130, 70), (256, 256, 128), (257, 129, 200),
+          (31, 300, 1023)]
+
+
+def exact_kind(types):
+    return O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    return gpu_util
+
+
+@pytest.mark.parametrize("types", ALL_TYPES)
+@pytest.mark.parametrize("rung", VALU_RUNGS + (MFMA,))
+def test_bit_exact_all_layouts_and_shapes(G, types, rung):
+    """int8 full range / integer-valued floats: any summation order must give the oracle's bits."""
+    for (la, lb), (m, n, k), (al, be) in itertools.product(LAYOUTS, SHAPES, [(1, 0), (2, -1)]):
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=m + 3 * n + 7 * k)
+        print("case", types, rung, la, lb, m, n, k, al, be, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, al, be, rung)
+        ref = O.gemm(types, a, b, c, m, n, k, la, lb, al, be)
+        assert np.array_equal(got, ref), (types, rung, la, lb, m, n, k, al, be)
+
+
+@pytest.mark.parametrize("types", ALL_TYPES[1:])
+@pytest.mark.parametrize("rung", VALU_RUNGS)
+def test_valu_rungs_sum_in_k_order(G, types, rung):
+    """Rungs 0-3 add each output's products in k order, so even N(0,1) data matches the oracle bit for bit."""
+    for (la, lb), (m, n, k) in itertools.product(LAYOUTS, [(65, 63, 129), (128, 192, 257)]):
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_NORMAL, seed=11)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1.0, 0.5, rung)
+        ref = O.gemm(types, a, b, c, m, n, k, la, lb, 1.0, 0.5)
+        assert np.array_equal(got, ref), (types, rung, la, lb, m, n, k)
+
+
+@pytest.mark.parametrize("types", ALL_TYPES[1:])
+def test_mfma_within_tolerance_on_normal_data(G, types):
+    """Blocked fp32 accumulation differs from the sequential sum only by rounding: <= 1e-3 (fp32 out) / 1e-2 (16-bit out)."""
+    for (la, lb), (m, n, k), variant in itertools.product(LAYOUTS, [(256, 256, 512), (300, 200, 1000)], (0, 1, 2)):
+        kind = O.FILL_UNIFORM_PM1 if types == O.F16F16F16 else O.FILL_NORMAL
+        a, b, c = O.make_inputs(types, m, n, k, kind=kind, seed=21)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1.0, 1.0, MFMA, variant)
+        truth, _ = O.gemm_f64(types, a, b, c, m, n, k, la, lb, 1.0, 1.0)
+        G.assert_within(types, got, truth, f"mfma vs fp64 truth {types} {la}{lb} {m}x{n}x{k} v{variant}")
+        ref = O.out_to_f64(types, O.gemm(types, a, b, c, m, n, k, la, lb, 1.0, 1.0))
+        G.assert_within(types, got, ref, "mfma vs sequential fp32 oracle")
+
+
+@pytest.mark.parametrize("types", ALL_TYPES)
+def test_mfma_every_variant_bit_exact(G, types):
+    nvar = G.capi.variant_count(types, G.capi.RUNG_MFMA)
+    assert nvar >= 3
+    for variant, (la, lb), (m, n, k) in itertools.product(range(1, nvar + 1), [(0, 1), (0, 0), (1, 0)],
+                                                          [(512, 512, 256), (300, 520, 130)]):
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=variant)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1, 1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 1, 1)), (types, variant, la, lb, m, n, k)
+
+
+@pytest.mark.parametrize("types", ALL_TYPES[1:])
+def test_skinny_rung(G, types):
+    for (m, n, k), (al, be) in itertools.product([(1, 16, 64), (1, 1000, 256), (8, 14336, 512), (16, 250, 128),
+                                                  (17, 33, 192), (32, 512, 4096)], [(1, 0), (0.5, 2)]):
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=5)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, al, be, SKINNY)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, al, be)), (types, m, n, k)
+        # decode-like data: activations N(0,1), weights N(0, 0.02)
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_NORMAL, seed=6, scale_b=0.02)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 0, G.capi.RUNG_AUTO)  # AUTO picks the same kernel
+        assert G.capi.plan(types, m, n, k, O.ROW, O.COL).rung == SKINNY
+        truth, _ = O.gemm_f64(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 0)
+        G.assert_within(types, got, truth, f"skinny {types} {m}x{n}x{k}")
+
+
+def test_skinny_rung_refuses_what_it_cannot_do(G):
+    a = torch.zeros(64 * 64, dtype=torch.int16, device="cuda")
+    for kw in (dict(m=33), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32)):
+        args = dict(types=O.BF16BF16BF16, m=8, n=64, k=64, la=O.ROW, lb=O.COL)
+        args.update(kw)
+        with pytest.raises(G.capi.GzError) as e:
+            G.capi.gemm(args["types"], a, a, None, a, args["m"], args["n"], args["k"], args["la"], args["lb"], 1, 0, SKINNY)
+        assert e.value.status == G.capi.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("types", ALL_TYPES)
+@pytest.mark.parametrize("rung", VALU_RUNGS + (MFMA,))
+def test_degenerate_and_unaligned(G, types, rung):
+    # K = 0: D = beta * C
+    m, n = 5, 9
+    a, b, c = O.make_inputs(types, m, n, 4, kind=exact_kind(types), seed=2)
+    got = G.run_gemm(types, a, b, c, m, n, 0, O.ROW, O.COL, 3, 2, rung)
+    assert np.array_equal(got, O.gemm(types, a, b, c, m, n, 0, O.ROW, O.COL, 3, 2))
+    # operands that start 1 element (not 16 bytes) into an allocation, tile-multiple shape
+    m, n, k = 256, 256, 256
+    a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=3)
+    for la, lb in LAYOUTS:
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1, 1, rung, misalign=1)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 1, 1)), (types, rung, la, lb)
+
+
+@pytest.mark.parametrize("types", ALL_TYPES)
+def test_beta_zero_never_reads_c(G, types):
+    m, n, k = 130, 70, 96
+    a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=4)
+    ref = O.gemm(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0)
+    poison = np.full(m * n, 0xFF, np.uint8).repeat(c.dtype.itemsize).view(c.dtype)  # NaN pattern for floats, -1 for int32
+    for rung in VALU_RUNGS + (MFMA,):
+        assert np.array_equal(G.run_gemm(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0, rung), ref)
+        assert np.array_equal(G.run_gemm(types, a, b, poison, m, n, k, O.ROW, O.COL, 1, 0, rung), ref)
+
+
+def test_int32_epilogue_wraps(G):
+    m = n = 64; k = 256
+    a = np.full(m * k, 127, np.int8); b = np.full(k * n, 127, np.int8); c = np.full(m * n, 2 ** 31 - 1, np.int32)
+    ref = O.gemm(O.S8S8S32, a, b, c, m, n, k, O.ROW, O.COL, 70000, 3)
+    for rung in VALU_RUNGS + (MFMA,):
+        assert np.array_equal(G.run_gemm(O.S8S8S32, a, b, c, m, n, k, O.ROW, O.COL, 70000, 3, rung), ref)
+
+
+def test_16bit_epilogue_rounding_order(G):
+    """The hand-built cases that pin the oracle's rounding order, on every rung."""
+    bf = lambda v: (np.asarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    k = 257
+    a = bf([1.0] * k); b = bf([1.0] * k)
+    for rung in VALU_RUNGS + (MFMA,):
+        d = G.run_gemm(O.BF16BF16BF16, a, b, None, 1, 1, k, O.ROW, O.COL, 1.5, 0.0, rung)
+        assert O.bf16_to_f32(d)[0, 0] == 384.0
+        d = G.run_gemm(O.BF16BF16BF16, bf([0.0]), bf([0.0]), bf([1.0078125]), 1, 1, 1, O.ROW, O.COL, 1.0, 1.0078125, rung)
+        assert O.bf16_to_f32(d)[0, 0] == 1.015625
