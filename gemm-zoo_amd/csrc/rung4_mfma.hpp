@@ -1,22 +1,31 @@
 // Rung 4: wavefront-level MFMA GEMM for gfx950.
 //
 // One work-group owns a BM x BN tile of D and walks K in slabs of 128 bytes per
-// row (64 16-bit elements or 128 int8).  Both operand slabs live in LDS as
-// [row][k] with a 16-byte pad per row (pitch 144 B), which makes the 128-bit
-// fragment reads of 16 consecutive rows hit 16 distinct 4-bank groups.
-// Each lane's MFMA operand is 16 contiguous K-bytes of one row, so a fragment
-// is a single ds_read_b128 whatever the element type:
+// row (64 16-bit elements or 128 int8).  Each lane's MFMA operand is 16
+// contiguous K-bytes of one row, so a fragment is a single ds_read_b128 whatever
+// the element type:
 //     v_mfma_f32_32x32x16_{bf16,f16}  (8 elements / lane)
 //     v_mfma_i32_32x32x32_i8          (16 elements / lane)
-// Operands whose contiguous dimension is not K (row-major B, column-major A)
-// are transposed in registers on their way into LDS.
 // The B fragment is passed as the instruction's first operand, so every lane
 // ends up with 4 consecutive columns of one output row and the epilogue stores
 // are 128-bit (fp32 / int32) or 64-bit (16-bit outputs).
 //
+// Three kernels share that tiling:
+//   mfma_gemm_kernel  general: any layout, any shape (predicated EDGE instantiation), any alignment.
+//                     Slabs are staged global -> registers -> LDS ([row][k], pitch 144 B: the 16-byte pad
+//                     makes the fragment reads of 16 consecutive rows hit 16 distinct 4-bank groups);
+//                     operands whose contiguous dimension is not K (row-major B, column-major A) are
+//                     transposed in registers on the way in.
+//   mfma_dtl_kernel   fast path for K-contiguous operands, whole tiles, 16-byte alignment: slabs go
+//                     global -> LDS directly (global_load_lds_dwordx4), unpadded swizzled rows.
+//   mfma_asm_kernel   the same data movement with a hand-placed instruction sequence (variant 5).
+//
 // Stands in for nvidia/kernels/sm_80/{bf16,fp16}_mma_gemm.cuh and
 // intel/kernels/xe_gemm_*_m8k16.hpp (same operation, new design).
 #pragma once
+#include <type_traits>
+#include <utility>
+
 #include "gz_common.hpp"
 #include "gz_mfma_cfg.hpp"
 
@@ -225,44 +234,67 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 
   const int ktiles = (g.K + BK - 1) / BK;
 
-  sa.load(g.A, g.M, g.K, m0, 0, tid);
-  sb.load(g.B, g.N, g.K, n0, 0, tid);
-  sa.store(lds, tid);
-  sb.store(lds + A_BYTES, tid);
-  __syncthreads();
-
   // fragment base offsets of this lane inside a stage
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
   const int a_off = (wm * WM + frag_row) * PITCH + frag_k;
   const int b_off = A_BYTES + (wn * WN + frag_row) * PITCH + frag_k;
 
+  // Two fragment sets: while the MFMAs of one K step run, the ds_reads of the next are in flight.
+  u32x4_t af[2][FM], bf[2][FN];
+  auto read_frags = [&](int set, const char* stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+      af[set][i] = *reinterpret_cast<const u32x4_t*>(stage + a_off + i * 32 * PITCH + ks * 32);
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+      bf[set][j] = *reinterpret_cast<const u32x4_t*>(stage + b_off + j * 32 * PITCH + ks * 32);
+  };
+  auto mma = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+      for (int j = 0; j < FN; j++) acc[i][j] = mfma32<TYPES>(bf[set][j], af[set][i], acc[i][j]);
+  };
+
+  // Prologue: slab 0 into LDS, slab 1 parked in registers, fragments of (slab 0, step 0) requested.
+  sa.load(g.A, g.M, g.K, m0, 0, tid);
+  sb.load(g.B, g.N, g.K, n0, 0, tid);
+  sa.store(lds, tid);
+  sb.store(lds + A_BYTES, tid);
+  if (ktiles > 1) {
+    sa.load(g.A, g.M, g.K, m0, BK, tid);
+    sb.load(g.B, g.N, g.K, n0, BK, tid);
+  }
+  __syncthreads();
+  read_frags(0, lds, 0);
+
+  // Steady state per slab (KSTEPS = 4 MFMA steps):
+  //   step 0..2 : request the fragments of the next step, then issue this step's MFMAs
+  //   after step 2: park registers (slab kt+1) -> other LDS buffer, request slab kt+2 from global memory
+  //   barrier     : every wave has written the other buffer and has finished reading this one
+  //   step 3     : request (slab kt+1, step 0) fragments from the other buffer, issue step 3 MFMAs
+  // so every LDS and global latency is covered by MFMAs, with one barrier per slab.
   for (int kt = 0; kt < ktiles; kt++) {
     const char* cur = lds + (kt & 1) * STAGE_BYTES;
     char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
-    const bool more = kt + 1 < ktiles;
-    if (more) {
-      sa.load(g.A, g.M, g.K, m0, (kt + 1) * BK, tid);
-      sb.load(g.B, g.N, g.K, n0, (kt + 1) * BK, tid);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS - 1; ks++) {
+      read_frags((ks + 1) & 1, cur, ks + 1);
+      mma(ks & 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-      u32x4_t af[FM], bf[FN];
-#pragma unroll
-      for (int i = 0; i < FM; i++)
-        af[i] = *reinterpret_cast<const u32x4_t*>(cur + a_off + i * 32 * PITCH + ks * 32);
-#pragma unroll
-      for (int j = 0; j < FN; j++)
-        bf[j] = *reinterpret_cast<const u32x4_t*>(cur + b_off + j * 32 * PITCH + ks * 32);
-#pragma unroll
-      for (int i = 0; i < FM; i++)
-#pragma unroll
-        for (int j = 0; j < FN; j++) acc[i][j] = mfma32<TYPES>(bf[j], af[i], acc[i][j]);
-    }
-    if (more) {
+    if (kt + 1 < ktiles) {
       sa.store(nxt, tid);
       sb.store(nxt + A_BYTES, tid);
     }
+    if (kt + 2 < ktiles) {
+      sa.load(g.A, g.M, g.K, m0, (kt + 2) * BK, tid);
+      sb.load(g.B, g.N, g.K, n0, (kt + 2) * BK, tid);
+    }
     __syncthreads();
+    if (kt + 1 < ktiles) read_frags(KSTEPS & 1, nxt, 0);
+    mma((KSTEPS - 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // Epilogue.  acc[i][j][4*q + e] is D(m, n + e) with
@@ -298,10 +330,425 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 }
 
 // ---------------------------------------------------------------------------
+// Fast path: both operands K-contiguous, whole tiles, 16-byte aligned.
+//
+// Global memory is copied straight into LDS by global_load_lds_dwordx4 (no
+// staging registers, no ds_write): one wave instruction moves 8 tile rows x 128
+// bytes and the hardware lays the 64 lanes' 16-byte chunks down contiguously, so
+// LDS rows are unpadded.  Bank conflicts are avoided by permuting which global
+// chunk each lane fetches: chunk c of tile row r lives at position
+//     p = c ^ swz(r),   swz(r) = (r & 7) ^ ((r >> 3) & 1)
+// which spreads any 8 consecutive rows over the 8 chunk columns and any 16
+// consecutive rows over both 128-byte halves of a 64-bank line.
+// ---------------------------------------------------------------------------
+__device__ inline int dtl_swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
+    mfma_dtl_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
+  using T = Traits<TYPES>;
+  using in_t = typename T::in_t;
+  using out_t = typename T::out_t;
+  using acc_v = typename AccVec<TYPES>::type;
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int ES = (int)sizeof(in_t);
+  constexpr int EPV = 16 / ES;
+  constexpr int BK = SLAB_BYTES / ES;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int FM = WM / 32, FN = WN / 32;
+  constexpr int ROWB = SLAB_BYTES;  // unpadded LDS row
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_PW = BM / 8 / NW, B_PW = BN / 8 / NW;  // 1 KiB copy instructions per wave and slab
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide over the waves");
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int K = g.K;
+
+  // ---- copy addressing: lane -> (row lr of an 8-row group, LDS position lp) ----
+  const int lr = lane >> 3, lp = lane & 7;
+  // the 8-row group index q = wave*PW + t has the parity of t when PW is even; (wave*PW)&1 covers odd PW
+  const in_t* a_src[2];
+  const in_t* b_src[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const int ca = lp ^ lr ^ (((wave * A_PW) & 1) ^ par);
+    const int cb = lp ^ lr ^ (((wave * B_PW) & 1) ^ par);
+    a_src[par] = g.A + (size_t)(m0 + 8 * wave * A_PW + lr) * K + ca * EPV;
+    b_src[par] = g.B + (size_t)(n0 + 8 * wave * B_PW + lr) * K + cb * EPV;
+  }
+  auto copy_slab = [&](char* stage, int k0) {
+#pragma unroll
+    for (int t = 0; t < A_PW; t++)
+      __builtin_amdgcn_global_load_lds((gptr_t)(a_src[t & 1] + (size_t)(8 * t) * K + k0),
+                                       (lptr_t)(stage + (wave * A_PW + t) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int t = 0; t < B_PW; t++)
+      __builtin_amdgcn_global_load_lds((gptr_t)(b_src[t & 1] + (size_t)(8 * t) * K + k0),
+                                       (lptr_t)(stage + A_BYTES + (wave * B_PW + t) * 1024), 16, 0, 0);
+  };
+
+  // ---- fragment addressing ----
+  const int frag_row = lane & 31, half = lane >> 5;
+  const int sw = dtl_swz(frag_row);
+  int pos[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) pos[ks] = ((ks * 2 + half) ^ sw) * 16;
+  const int a_base = (wm * WM + frag_row) * ROWB;
+  const int b_base = A_BYTES + (wn * WN + frag_row) * ROWB;
+
+  acc_v acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; i++)
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+
+  u32x4_t af[2][FM], bf[2][FN];
+  auto read_frags = [&](int set, const char* stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+      af[set][i] = *reinterpret_cast<const u32x4_t*>(stage + a_base + i * 32 * ROWB + pos[ks]);
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+      bf[set][j] = *reinterpret_cast<const u32x4_t*>(stage + b_base + j * 32 * ROWB + pos[ks]);
+  };
+  auto mma = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+      for (int j = 0; j < FN; j++) acc[i][j] = mfma32<TYPES>(bf[set][j], af[set][i], acc[i][j]);
+  };
+
+  const int ktiles = K / BK;  // >= 1 on this path
+  copy_slab(lds, 0);
+  if (ktiles > 1) copy_slab(lds + STAGE_BYTES, BK);
+  if (ktiles > 1) __builtin_amdgcn_s_waitcnt(0x0F70 | ((A_PW + B_PW) & 15) | (((A_PW + B_PW) >> 4) << 14));
+  else __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  read_frags(0, lds, 0);
+
+  // One barrier per slab.  At the barrier of slab kt every wave has finished reading buffer kt&1 and the
+  // copies of slab kt+1 have landed, so the copies of slab kt+2 may overwrite buffer kt&1 right after it;
+  // they then have a whole slab of MFMAs to complete.
+  for (int kt = 0; kt < ktiles; kt++) {
+    char* cur = lds + (kt & 1) * STAGE_BYTES;
+    char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS - 1; ks++) {
+      read_frags((ks + 1) & 1, cur, ks + 1);
+      mma(ks & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my copies landed, my fragment reads returned
+    __syncthreads();
+    if (kt + 2 < ktiles) copy_slab(cur, (kt + 2) * BK);
+    if (kt + 1 < ktiles) read_frags(KSTEPS & 1, nxt, 0);
+    mma((KSTEPS - 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // Epilogue: same register layout as the staged kernel.
+  const int N = g.N;
+  const bool use_c = g.beta != 0;
+#pragma unroll
+  for (int i = 0; i < FM; i++) {
+    const int m = m0 + wm * WM + 32 * i + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
+        const size_t o = (size_t)m * N + n;
+        out_t cv[4] = {0, 0, 0, 0}, dv[4];
+        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+#pragma unroll
+        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Hand-scheduled fast path.
+//
+// Same data movement as mfma_dtl_kernel (direct-to-LDS copies, swizzled unpadded rows, two LDS buffers, one
+// barrier per slab), but the main loop is a fixed instruction sequence: a wavefront issues in order, so one
+// memory instruction is placed after each MFMA and nowhere else.  Measured on MI355X, 16 MFMAs with 8
+// ds_read_b128 and 4 LDS copies slotted in this way run at the rate of 16 bare MFMAs, while the same
+// instructions bunched together (the compiler's order) cost 40-50 % more.  The sequence is written as
+// volatile asm statements so that neither the scheduler nor the wait-count pass (which, with an LDS copy
+// pending, waits for lgkmcnt(0) before the first MFMA of every step) can change it; all s_waitcnt are
+// placed by hand:
+//   step start : lgkmcnt(0)  - the fragments of this step were requested one step (>= 8 MFMAs) ago
+//   barrier    : vmcnt(0) lgkmcnt(0) - this wave's copies of the next slab have landed, its reads of the
+//                current buffer have returned
+// Per slab (4 steps): step 0..2 read the next step's fragments from the current buffer, step 3 (after the
+// barrier) reads step 0 of the next slab from the other buffer.  The copies of slab kt+2 into the buffer
+// freed by that barrier are issued in step 3 of slab kt and step 0 of slab kt+1, so they have two more
+// steps to land.
+// ---------------------------------------------------------------------------
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F> __device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <int OFF> __device__ __forceinline__ void asm_ds_read16(u32x4_t& dst, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
+}
+// LDS destination base of the following copies.  Writing M0 waits for the copies already queued to read it,
+// which can hold up the wave's whole instruction stream, so it is written once per group of copies; the copies
+// of a group step through LDS with their immediate offset.
+__device__ __forceinline__ void asm_set_m0(uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory");
+}
+// 64 lanes x 16 bytes from sbase + voff + OFF (per lane) to LDS at M0 + OFF + 16 * lane: the immediate offset
+// applies to both addresses, so the caller passes the source base minus OFF.
+template <int OFF> __device__ __forceinline__ void asm_copy16(uint32_t voff, const void* sbase_minus_off) {
+  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
+  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase_minus_off), "i"(OFF) : "memory");
+}
+template <int TYPES>
+__device__ __forceinline__ void asm_mfma32(typename AccVec<TYPES>::type& c, const u32x4_t& first, const u32x4_t& second) {
+  if constexpr (TYPES == GZ_S8S8S32)
+    asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
+  else if constexpr (TYPES == GZ_F16F16F16)
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
+  else
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
+}
+
+// orders later reads of an accumulator after every asm statement that precedes this one
+template <int TYPES> __device__ __forceinline__ void asm_touch_acc(typename AccVec<TYPES>::type& c) {
+  asm volatile("" : "+a"(c));
+}
+
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
+    mfma_asm_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
+  using T = Traits<TYPES>;
+  using in_t = typename T::in_t;
+  using out_t = typename T::out_t;
+  using acc_v = typename AccVec<TYPES>::type;
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int ES = (int)sizeof(in_t);
+  constexpr int EPV = 16 / ES;
+  constexpr int BK = SLAB_BYTES / ES;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int FM = WM / 32, FN = WN / 32;
+  constexpr int ROWB = SLAB_BYTES;
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_PW = BM / 8 / NW, B_PW = BN / 8 / NW;
+  constexpr int NCP = A_PW + B_PW, NMMA = FM * FN, NRD = FM + FN;
+  static_assert(A_PW <= 8 && B_PW <= 8 && A_PW % 2 == 0 && B_PW % 2 == 0, "a copy group must fit the immediate offset range");
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide over the waves");
+  static_assert(KSTEPS == 4, "the step schedule below is written for four MFMA steps per slab");
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int K = g.K;
+
+  // ---- copy addressing (see mfma_dtl_kernel) ----
+  const int lr = lane >> 3, lp = lane & 7;
+  uint32_t a_voff[2], b_voff[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const int ca = lp ^ lr ^ (((wave * A_PW) & 1) ^ par);
+    const int cb = lp ^ lr ^ (((wave * B_PW) & 1) ^ par);
+    a_voff[par] = (uint32_t)((lr * K + ca * EPV) * ES);
+    b_voff[par] = (uint32_t)((lr * K + cb * EPV) * ES);
+  }
+  const char* a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(m0 + 8 * wave * A_PW) * K * ES;
+  const char* b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 8 * wave * B_PW) * K * ES;
+  const size_t group_step = (size_t)8 * K * ES;
+  // copy number C of the slab that starts at K byte `kbyte`: copies [0, A_PW) move this wave's A rows, the rest
+  // its B rows.  Each group has one M0 (set by copy_group_begin) in the middle of its LDS span.
+  auto copy_group_begin = [&](auto c_c, int st) {
+    constexpr int C = decltype(c_c)::value;
+    if constexpr (C == 0) asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024);
+    else if constexpr (C == A_PW) asm_set_m0(lds_base + st * STAGE_BYTES + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024);
+  };
+  auto copy_one = [&](auto c_c, int st, size_t kbyte) {
+    constexpr int C = decltype(c_c)::value;
+    copy_group_begin(c_c, st);
+    if constexpr (C < A_PW) {
+      constexpr int OFF = (C - A_PW / 2) * 1024;
+      asm_copy16<OFF>(a_voff[C & 1], a_ubase + C * group_step + kbyte - OFF);
+    } else {
+      constexpr int Tn = C - A_PW;
+      constexpr int OFF = (Tn - B_PW / 2) * 1024;
+      asm_copy16<OFF>(b_voff[Tn & 1], b_ubase + Tn * group_step + kbyte - OFF);
+    }
+  };
+
+  // ---- fragment addressing ----
+  const int frag_row = lane & 31, half = lane >> 5;
+  const int sw = dtl_swz(frag_row);
+  uint32_t a_addr[2][KSTEPS], b_addr[2][KSTEPS];
+#pragma unroll
+  for (int st = 0; st < 2; st++)
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      const int pos = ((ks * 2 + half) ^ sw) * 16;
+      a_addr[st][ks] = lds_base + st * STAGE_BYTES + (wm * WM + frag_row) * ROWB + pos;
+      b_addr[st][ks] = lds_base + st * STAGE_BYTES + A_BYTES + (wn * WN + frag_row) * ROWB + pos;
+    }
+
+  acc_v acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; i++)
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+  // the zeroing above is ordinary code: pin it before the asm sequence (and give the VALU writes their wait
+  // states before an MFMA may read the accumulators)
+  static_for<NMMA>([&](auto q_c) {
+    constexpr int Q = decltype(q_c)::value;
+    asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
+  });
+  asm volatile("s_nop 7" ::: "memory");
+  u32x4_t af[2][FM], bf[2][FN];
+
+  // fragment read number R (A fragments first) of K step `ks` of buffer `st` into register set SET
+  auto read_one = [&](auto set_c, auto r_c, int st, int ks) {
+    constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value;
+    if constexpr (R < FM) asm_ds_read16<R * 32 * ROWB>(af[SET][R], a_addr[st][ks]);
+    else asm_ds_read16<(R - FM) * 32 * ROWB>(bf[SET][R - FM], b_addr[st][ks]);
+  };
+
+  // One MFMA step.  P: step within the slab; CUR: buffer of the slab.  The fragments of the next step are always
+  // requested (past the last slab they are stale data that nobody multiplies); `copy` says whether this step's
+  // quarter of the LDS copies is issued - a uniform run-time branch around a copy does not disturb the
+  // sequence, and one code path for every slab keeps the accumulators in the same registers throughout.
+  auto step = [&](auto p_c, auto cur_c, bool copy, int kt) {
+    constexpr int P = decltype(p_c)::value, CUR = decltype(cur_c)::value;
+    constexpr int SET = P & 1;
+    constexpr int RST = P < 3 ? CUR : (CUR ^ 1), RKS = P < 3 ? P + 1 : 0;
+    // copies: step 3 -> first quarter of slab kt+2 into CUR ; steps 0, 1, 2 -> the other quarters of slab kt+1
+    // into CUR^1 (the texture path needs most of a slab's time to move a slab, so the copies are spread evenly)
+    constexpr int QN = (P + 1) & 3;  // quarter number: step 3 -> 0, step 0 -> 1, step 1 -> 2, step 2 -> 3
+    constexpr int CB = QN * NCP / 4, CE = (QN + 1) * NCP / 4;
+    constexpr int NC = CE - CB;
+    constexpr int NOPS = NRD + NC;
+    const int cst = P == 3 ? CUR : (CUR ^ 1);
+    const size_t kbyte = (size_t)(kt + (P == 3 ? 2 : 1)) * SLAB_BYTES;
+    asm volatile("s_waitcnt lgkmcnt(0)");
+    static_for<NMMA>([&](auto q_c) {
+      constexpr int Q = decltype(q_c)::value;
+      asm_mfma32<TYPES>(acc[Q / FN][Q % FN], bf[SET][Q % FN], af[SET][Q / FN]);
+      static_for<NOPS>([&](auto o_c) {
+        constexpr int O = decltype(o_c)::value;
+        constexpr int SLOT = NOPS <= NMMA ? O : (O * NMMA) / NOPS;
+        if constexpr (SLOT == Q) {
+          if constexpr (O < NRD) {
+            read_one(std::integral_constant<int, SET ^ 1>{}, o_c, RST, RKS);
+          } else {
+            if (copy) copy_one(std::integral_constant<int, CB + O - NRD>{}, cst, kbyte);
+          }
+        }
+      });
+    });
+  };
+
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+
+  // One slab: steps 0..2 from buffer CUR, barrier, step 3.
+  //   steps 0..2 issue quarters 1..3 of the copies of slab kt+1 (slab 1 was copied whole by the prologue)
+  //   step 3 issues quarter 0 of the copies of slab kt+2
+  auto slab = [&](auto cur_c, int kt, int ktiles) {
+    const bool later = kt >= 1 && kt + 1 < ktiles, first = kt + 2 < ktiles;
+    step(I0{}, cur_c, later, kt);
+    step(I1{}, cur_c, later, kt);
+    step(I2{}, cur_c, later, kt);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    step(I3{}, cur_c, first, kt);
+  };
+
+  const int ktiles = K / BK;  // >= 1 on this path
+  // Prologue: slab 0 and slab 1 copied whole; fragments of (slab 0, step 0) requested.
+  static_for<NCP>([&](auto c) { copy_one(c, 0, 0); });
+  if (ktiles > 1) static_for<NCP>([&](auto c) { copy_one(c, 1, (size_t)SLAB_BYTES); });
+  if (ktiles > 1) {
+    if constexpr (NCP == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (NCP == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  asm volatile("s_barrier" ::: "memory");
+  static_for<NRD>([&](auto r) { read_one(I0{}, r, 0, 0); });
+
+  // Two slabs per trip so that the buffer index is a compile-time constant; the second one is skipped (not
+  // duplicated) when K has an odd number of slabs.
+  for (int kt = 0; kt < ktiles; kt += 2) {
+    slab(I0{}, kt, ktiles);
+    if (kt + 1 < ktiles) slab(I1{}, kt + 1, ktiles);
+  }
+  // The last MFMAs must have written their accumulators before ordinary code reads them: the hazard
+  // recogniser does not look inside asm statements, so the wait states are spelled out, and every
+  // accumulator is passed through an (empty) asm placed after them so that no read can be hoisted above.
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7" ::: "memory");
+  static_for<NMMA>([&](auto q_c) {
+    constexpr int Q = decltype(q_c)::value;
+    asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
+  });
+
+  // Epilogue: same register layout as the staged kernel.
+  const int N = g.N;
+  const bool use_c = g.beta != 0;
+#pragma unroll
+  for (int i = 0; i < FM; i++) {
+    const int m = m0 + wm * WM + 32 * i + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
+        const size_t o = (size_t)m * N + n;
+        out_t cv[4] = {0, 0, 0, 0}, dv[4];
+        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+#pragma unroll
+        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Launcher
 // ---------------------------------------------------------------------------
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
-static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, hipStream_t s) {
+static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, bool hand_scheduled, hipStream_t s) {
   const int tiles_m = ceil_div(g.M, BM), tiles_n = ceil_div(g.N, BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(WAVES_M * WAVES_N * 64);
   const size_t lds = 2u * (size_t)(BM + BN) * PITCH;
@@ -315,6 +762,25 @@ static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, hipStream_t s) {
     hipLaunchKernelGGL(kern, grid, block, lds, s, g, tiles_m, tiles_n);                             \
   } while (0)
 
+  if (!edge && akc && bkc) {  // whole tiles, K-contiguous operands, aligned: direct-to-LDS fast path
+    const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
+    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
+      if (hand_scheduled) {
+        auto kern = mfma_asm_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
+        GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)dlds));
+        hipLaunchKernelGGL(kern, grid, block, dlds, s, g, tiles_m, tiles_n);
+        GZ_HIP_TRY(hipGetLastError());
+        return GZ_OK;
+      }
+    }
+    auto kern = mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
+    GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)dlds));
+    hipLaunchKernelGGL(kern, grid, block, dlds, s, g, tiles_m, tiles_n);
+    GZ_HIP_TRY(hipGetLastError());
+    return GZ_OK;
+  }
   if (edge) {
     if (akc && bkc) GZ_LAUNCH(true, true, true);
     else if (akc && !bkc) GZ_LAUNCH(true, false, true);
@@ -341,10 +807,11 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipS
   const bool edge = mfma_needs_edge(cfg, (int)sizeof(in_t), (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N,
                                     g.K, g.A, g.B, g.C, g.D);
   switch (cfg.id) {
-    case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, s);
-    case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, s);
-    case 3: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, s);
-    case 4: return launch_cfg<TYPES, 256, 128, 2, 2>(g, edge, s);
+    case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, false, s);
+    case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, false, s);
+    case 3: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, false, s);
+    case 4: return launch_cfg<TYPES, 256, 128, 2, 2>(g, edge, false, s);
+    case 5: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, true, s);
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);
