@@ -10,7 +10,8 @@ struct MfmaCfg {
   int id;       // variant id (1-based; 0 means "let the launcher choose")
   int bm, bn;   // work-group tile
   int waves_m, waves_n;
-  int hand_scheduled;  // fast path uses the fixed instruction sequence instead of the compiler's schedule
+  int hand_scheduled;  // fast path: 0 compiler-scheduled, 1 fixed sequence / two 128-byte buffers,
+                       // 2 fixed sequence / four 64-byte buffers
 };
 
 // K slab per tile row is 128 bytes whatever the element type.
@@ -23,6 +24,8 @@ static const MfmaCfg kMfmaCfgs[] = {
     {3, 128, 128, 2, 2, 0},  // small tile for small problems / ragged tails
     {4, 256, 128, 2, 2, 0},  // 4 waves of 128x64
     {5, 256, 256, 2, 2, 1},  // tile of variant 1 with the hand-scheduled main loop
+    {6, 256, 256, 2, 2, 2},  // tile of variant 1, hand-scheduled, four-buffer pipeline
+    {7, 256, 256, 2, 4, 2},  // tile of variant 2 (8 waves), hand-scheduled, four-buffer pipeline
 };
 constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
 
@@ -40,9 +43,15 @@ inline bool mfma_resolve(int types, int M, int N, int /*K*/, int variant, int nu
   auto tiles = [&](const MfmaCfg& c) {
     return (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
   };
-  // measured on MI355X: with 16-bit inputs the 8-wave split of the big tile wins (bf16 4096^3: 129 us
-  // against 140 us), with int8 the 4-wave split does (8192^3: 651 us against 677 us)
-  if (tiles(kMfmaCfgs[0]) >= num_cus) *out = types == 0 ? kMfmaCfgs[0] : kMfmaCfgs[1];
+  // Measured on MI355X (interleaved runs, us): bf16 4096^3  v1 117  v2 109  v5 108  v6 109  v7 106
+  //                                           bf16 8192^3  v1 904  v2 865  v6 845  v7 885
+  //                                           int8 8192^3  v1 543  v2 558  v5 579  v6 536  v7 582
+  // The hand-scheduled kernels only exist for K-contiguous operands and whole tiles; on any other problem
+  // the same tile runs the general kernel, so choosing them here is always safe.
+  if (tiles(kMfmaCfgs[0]) >= num_cus) {
+    if (types == 0) *out = kMfmaCfgs[5];                                  // int8: 4 waves, four-buffer pipeline
+    else *out = tiles(kMfmaCfgs[0]) <= 2 * num_cus ? kMfmaCfgs[6] : kMfmaCfgs[5];
+  }
   else if (tiles(kMfmaCfgs[3]) >= num_cus) *out = kMfmaCfgs[3];
   else *out = kMfmaCfgs[2];
   return true;

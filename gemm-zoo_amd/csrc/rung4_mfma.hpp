@@ -744,11 +744,17 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   }
 }
 
+}  // namespace gz
+
+#include "rung4_mfma_pipe4.hpp"
+
+namespace gz {
+
 // ---------------------------------------------------------------------------
 // Launcher
 // ---------------------------------------------------------------------------
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
-static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, bool hand_scheduled, hipStream_t s) {
+static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, int hand_scheduled, hipStream_t s) {
   const int tiles_m = ceil_div(g.M, BM), tiles_n = ceil_div(g.N, BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(WAVES_M * WAVES_N * 64);
   const size_t lds = 2u * (size_t)(BM + BN) * PITCH;
@@ -764,8 +770,19 @@ static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, bool hand_scheduled, 
 
   if (!edge && akc && bkc) {  // whole tiles, K-contiguous operands, aligned: direct-to-LDS fast path
     const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
+    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+      if (hand_scheduled == 2) {
+        auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
+        const size_t plds = 4u * (size_t)(BM + BN) * 64;
+        GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)plds));
+        hipLaunchKernelGGL(kern, grid, block, plds, s, g, tiles_m, tiles_n);
+        GZ_HIP_TRY(hipGetLastError());
+        return GZ_OK;
+      }
+    }
     if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
-      if (hand_scheduled) {
+      if (hand_scheduled == 1) {
         auto kern = mfma_asm_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
         GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)dlds));
@@ -807,11 +824,13 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipS
   const bool edge = mfma_needs_edge(cfg, (int)sizeof(in_t), (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N,
                                     g.K, g.A, g.B, g.C, g.D);
   switch (cfg.id) {
-    case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, false, s);
-    case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, false, s);
-    case 3: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, false, s);
-    case 4: return launch_cfg<TYPES, 256, 128, 2, 2>(g, edge, false, s);
-    case 5: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, true, s);
+    case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
+    case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);
+    case 3: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 0, s);
+    case 4: return launch_cfg<TYPES, 256, 128, 2, 2>(g, edge, 0, s);
+    case 5: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 1, s);
+    case 6: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s);
+    case 7: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s);
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);

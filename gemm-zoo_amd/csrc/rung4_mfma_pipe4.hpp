@@ -1,0 +1,230 @@
+// MFMA rung, deep-pipeline fast path: four LDS buffers of 64-byte K rows.
+//
+// Why four buffers.  Moving a K slab from L2 into LDS takes the texture path most of the time the matrix
+// pipe needs to consume it, and a direct-to-LDS copy lands 1000-1500 cycles after it is issued.  With two
+// 128-byte buffers a copy can only start when its buffer has been drained and must have landed one slab
+// later, so either the copies are bunched right after the barrier (and the waves, which issue in order,
+// stall behind them) or the last ones are waited for.  Halving the K extent of a buffer (64 bytes per
+// row: 32 16-bit elements or 64 int8, two MFMA steps) and keeping four of them lets every copy be issued
+// evenly - four per wave and MFMA step - a full three half-slabs before its data is needed.
+//
+// Per half-slab h (buffer h % 4):
+//   step 0 : MFMAs on the fragments of (h, step 0); requests the fragments of (h, step 1);
+//            issues the B-row copies of half-slab h+3 into buffer (h+3) % 4
+//   barrier: lgkmcnt(0) - this wave has finished reading buffer h % 4, which is free afterwards;
+//            vmcnt(2n)  - this wave's copies of half-slab h+1 have landed (the 2n issued later may fly,
+//                         n = copies per wave and half-slab)
+//   step 1 : MFMAs on (h, step 1); requests the fragments of (h+1, step 0) from buffer (h+1) % 4;
+//            issues the A-row copies of half-slab h+4 into buffer h % 4
+// One memory instruction follows each MFMA; the sequence is fixed with asm statements (see mfma_asm_kernel).
+//
+// LDS rows are unpadded 64-byte rows; chunk c (16 bytes) of tile row r lives at position c ^ ((r >> 2) & 3),
+// which spreads 16 consecutive rows over the 16 four-bank groups of a 64-bank line.
+#pragma once
+
+namespace gz {
+
+__device__ inline int pipe4_swz(int r) { return (r >> 2) & 3; }
+
+// copy with a lane mask: an all-zero mask turns the instruction into a no-op that still takes its place in
+// the sequence (and in the vmcnt order)
+template <int OFF>
+__device__ __forceinline__ void asm_copy16_masked(uint32_t voff, const void* sbase_minus_off, uint64_t mask) {
+  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
+  asm volatile("s_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2\n\ts_mov_b64 exec, -1"
+               :
+               : "v"(voff), "s"(sbase_minus_off), "i"(OFF), "s"(mask)
+               : "memory");
+}
+
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
+    mfma_pipe4_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
+  using T = Traits<TYPES>;
+  using in_t = typename T::in_t;
+  using out_t = typename T::out_t;
+  using acc_v = typename AccVec<TYPES>::type;
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int ES = (int)sizeof(in_t);
+  constexpr int EPV = 16 / ES;
+  constexpr int ROWB = 64;            // K bytes per row and buffer
+  constexpr int HK = ROWB / ES;       // K elements per half-slab
+  constexpr int NST = 4;              // LDS buffers
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int FM = WM / 32, FN = WN / 32;
+  constexpr int NMMA = FM * FN, NRD = FM + FN;
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (16 rows) per wave and half-slab
+  constexpr int NCP = A_PW + B_PW;
+  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile rows must divide over the waves");
+  static_assert(A_PW <= 8 && B_PW <= 8 && A_PW % 2 == 0 && B_PW % 2 == 0, "a copy group must fit the immediate offset range");
+  static_assert(NCP == 8 || NCP == 4, "the vmcnt immediates below are written out for 8 or 4 copies per wave and half-slab");
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int K = g.K;
+  const int nh = K / HK;  // half-slabs, >= 2 on this path
+
+  // ---- copy addressing: lane -> (row lr of a 16-row group, LDS position lp) ----
+  const int lr = lane >> 2, lp = lane & 3;
+  const uint32_t voff = (uint32_t)((lr * K + (lp ^ pipe4_swz(lr)) * EPV) * ES);
+  const char* a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(m0 + 16 * wave * A_PW) * K * ES;
+  const char* b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 16 * wave * B_PW) * K * ES;
+  const size_t group_step = (size_t)16 * K * ES;
+  // A-row copies of half-slab hs into buffer st (one M0 for the group)
+  auto copy_a_begin = [&](int st) { asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024); };
+  auto copy_b_begin = [&](int st) {
+    asm_set_m0(lds_base + st * STAGE_BYTES + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024);
+  };
+  auto copy_a = [&](auto t_c, int hs, uint64_t mask) {
+    constexpr int Tn = decltype(t_c)::value, OFF = (Tn - A_PW / 2) * 1024;
+    asm_copy16_masked<OFF>(voff, a_ubase + Tn * group_step + (size_t)hs * ROWB - OFF, mask);
+  };
+  auto copy_b = [&](auto t_c, int hs, uint64_t mask) {
+    constexpr int Tn = decltype(t_c)::value, OFF = (Tn - B_PW / 2) * 1024;
+    asm_copy16_masked<OFF>(voff, b_ubase + Tn * group_step + (size_t)hs * ROWB - OFF, mask);
+  };
+
+  // ---- fragment addressing: one LDS byte address per (buffer, step) ----
+  const int frag_row = lane & 31, half = lane >> 5;
+  const int sw = pipe4_swz(frag_row);
+  uint32_t a_addr[NST][2], b_addr[NST][2];
+#pragma unroll
+  for (int st = 0; st < NST; st++)
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      const int pos = ((ks * 2 + half) ^ sw) * 16;
+      a_addr[st][ks] = lds_base + st * STAGE_BYTES + (wm * WM + frag_row) * ROWB + pos;
+      b_addr[st][ks] = lds_base + st * STAGE_BYTES + A_BYTES + (wn * WN + frag_row) * ROWB + pos;
+    }
+
+  acc_v acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; i++)
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+  static_for<NMMA>([&](auto q_c) {
+    constexpr int Q = decltype(q_c)::value;
+    asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
+  });
+  asm volatile("s_nop 7" ::: "memory");
+  u32x4_t af[2][FM], bf[2][FN];
+
+  auto read_one = [&](auto set_c, auto r_c, int st, int ks) {
+    constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value;
+    if constexpr (R < FM) asm_ds_read16<R * 32 * ROWB>(af[SET][R], a_addr[st][ks]);
+    else asm_ds_read16<(R - FM) * 32 * ROWB>(bf[SET][R - FM], b_addr[st][ks]);
+  };
+
+  // One MFMA step: NMMA MFMAs on register set SET; after MFMA q the q-th memory instruction of the step:
+  // first the NRD fragment reads of (buffer rst, step rks) into the other set, then this step's copies.
+  auto step = [&](auto set_c, int rst, int rks, auto copy_is_a, int cst, int chs, uint64_t cmask) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr bool IS_A = decltype(copy_is_a)::value;
+    constexpr int NC = IS_A ? A_PW : B_PW;
+    constexpr int NOPS = NRD + NC;
+    static_assert(NOPS <= NMMA, "one memory instruction per MFMA");
+    asm volatile("s_waitcnt lgkmcnt(0)");
+    if constexpr (IS_A) copy_a_begin(cst);
+    else copy_b_begin(cst);
+    static_for<NMMA>([&](auto q_c) {
+      constexpr int Q = decltype(q_c)::value;
+      asm_mfma32<TYPES>(acc[Q / FN][Q % FN], bf[SET][Q % FN], af[SET][Q / FN]);
+      if constexpr (Q < NRD) {
+        read_one(std::integral_constant<int, SET ^ 1>{}, q_c, rst, rks);
+      } else if constexpr (Q < NOPS) {
+        if constexpr (IS_A) copy_a(std::integral_constant<int, Q - NRD>{}, chs, cmask);
+        else copy_b(std::integral_constant<int, Q - NRD>{}, chs, cmask);
+      }
+    });
+  };
+
+  const std::true_type is_a{};
+  const std::false_type is_b{};
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  // lane mask of a copy as a scalar register pair: all ones while the half-slab exists, zero past the end
+  auto mask_if = [](bool on) -> uint64_t {
+    const uint32_t w = (uint32_t)__builtin_amdgcn_readfirstlane(on ? -1 : 0);
+    return ((uint64_t)w << 32) | w;
+  };
+
+  // ---- prologue: half-slabs 0, 1, 2 whole and the A rows of 3 ----
+  static_for<3>([&](auto h_c) {
+    constexpr int H = decltype(h_c)::value;
+    const uint64_t m = mask_if(H < nh);
+    copy_a_begin(H);
+    static_for<A_PW>([&](auto t) { copy_a(t, H, m); });
+    copy_b_begin(H);
+    static_for<B_PW>([&](auto t) { copy_b(t, H, m); });
+  });
+  copy_a_begin(3);
+  {
+    const uint64_t m3 = mask_if(3 < nh);
+    static_for<A_PW>([&](auto t) { copy_a(t, 3, m3); });
+  }
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");  // simple and safe: the prologue is short
+  static_for<NRD>([&](auto r) { read_one(I0{}, r, 0, 0); });
+
+  // ---- one half-slab; S = h % 4 at compile time ----
+  auto half_slab = [&](auto s_c, int h) {
+    constexpr int S = decltype(s_c)::value;
+    step(I0{}, S, 1, is_b, (S + 3) % NST, h + 3, mask_if(h + 3 < nh));
+    if (h + 3 < nh) {  // the 2 * NCP copies issued after those of half-slab h+1 may stay in flight
+      if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    step(I1{}, (S + 1) % NST, 0, is_a, S, h + 4, mask_if(h + 4 < nh));
+  };
+
+  for (int h = 0; h < nh; h += 4) {
+    half_slab(std::integral_constant<int, 0>{}, h);
+    if (h + 1 < nh) half_slab(std::integral_constant<int, 1>{}, h + 1);
+    if (h + 2 < nh) half_slab(std::integral_constant<int, 2>{}, h + 2);
+    if (h + 3 < nh) half_slab(std::integral_constant<int, 3>{}, h + 3);
+  }
+
+  // no copy may still be in flight when the work-group ends, and the last MFMAs must have written their
+  // accumulators before ordinary code reads them
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_nop 7" ::: "memory");
+  static_for<NMMA>([&](auto q_c) {
+    constexpr int Q = decltype(q_c)::value;
+    asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
+  });
+
+  // Epilogue: same register layout as the staged kernel.
+  const int N = g.N;
+  const bool use_c = g.beta != 0;
+#pragma unroll
+  for (int i = 0; i < FM; i++) {
+    const int m = m0 + wm * WM + 32 * i + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
+        const size_t o = (size_t)m * N + n;
+        out_t cv[4] = {0, 0, 0, 0}, dv[4];
+        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+#pragma unroll
+        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+      }
+    }
+  }
+}
+
+}  // namespace gz
