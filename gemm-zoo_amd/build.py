@@ -89,11 +89,30 @@ def build_comparator(verbose=True):
     return target
 
 
+def build_benches(verbose=True, jobs=8):
+    """The C++ drivers under bench/ (gemm-zoo's bench mains on the functor surface) -> bench/bin/."""
+    bench_dir = HERE / "bench"
+    out_dir = bench_dir / "bin"
+    out_dir.mkdir(exist_ok=True)
+    include = HERE.parent / "include"
+
+    def one(src: Path):
+        exe = out_dir / src.stem
+        _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",
+              f"-I{include}", str(src), "-o", str(exe), f"-L{LIB}", "-lgemmzoo", "-lgemmzoo_hipblaslt",
+              "-Wl,-rpath,$ORIGIN/../../lib", "-Wl,-rpath,/opt/rocm/lib"])
+        return exe
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        return list(ex.map(one, sorted(bench_dir.glob("*.cpp"))))
+
+
 def build_all(verbose=True):
     out = [build_product(verbose)]
     cmp_lib = build_comparator(verbose)
     if cmp_lib:
         out.append(cmp_lib)
+        out.extend(build_benches(verbose))
     return out
 
 

@@ -26,7 +26,7 @@ OUT_SIZE = {S8S8S32: 4, BF16BF16F32: 4, BF16BF16BF16: 2, F16F16F16: 2}
 
 EXPORTS = [
     "gz_gemm_s8s8s32", "gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16", "gz_gemm",
-    "gz_plan", "gz_variant_count", "gz_rung_name", "gz_types_name", "gz_fill", "gz_compare",
+    "gz_plan", "gz_variant_count", "gz_rung_name", "gz_types_name", "gz_fill", "gz_compare", "gz_compare_rel",
     "gz_last_error", "gz_version",
 ]
 
@@ -73,6 +73,7 @@ def _load():
     lib.gz_types_name.restype = C.c_char_p
     lib.gz_fill.argtypes = [vp, i64, i32, i32, f32, C.c_uint64, vp]
     lib.gz_compare.argtypes = [vp, vp, i64, i32, f32, C.POINTER(C.c_int64), vp]
+    lib.gz_compare_rel.argtypes = [vp, vp, i64, i32, f32, f32, C.POINTER(C.c_int64), vp]
     lib.gz_last_error.restype = C.c_char_p
     for name in EXPORTS:
         fn = getattr(lib, name)
@@ -125,10 +126,11 @@ def fill(dst, count: int, dtype: int, kind: int, scale: float = 1.0, seed: int =
     check(lib.gz_fill(_ptr(dst), count, dtype, kind, scale, seed, stream))
 
 
-def compare(out, ref, count: int, dtype: int, abs_threshold: float = 0.0, stream: int = 0) -> int:
+def compare(out, ref, count: int, dtype: int, abs_threshold: float = 0.0, stream: int = 0,
+            rel_threshold: float = 0.0) -> int:
     """Returns the number of differing elements (0 = equal); raises only on API errors."""
     nd = C.c_int64(0)
-    st = lib.gz_compare(_ptr(out), _ptr(ref), count, dtype, abs_threshold, C.byref(nd), stream)
+    st = lib.gz_compare_rel(_ptr(out), _ptr(ref), count, dtype, abs_threshold, rel_threshold, C.byref(nd), stream)
     if st not in (OK, ERR_MISMATCH):
         raise GzError(st, last_error())
     return nd.value

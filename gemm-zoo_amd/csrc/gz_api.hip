@@ -238,8 +238,8 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
     }
     case GZ_RUNG_SKINNY: {
       if (!skinny_supported(types, m, n, k, layoutA, layoutB)) {
-        set_error("skinny rung needs a 16-bit float type, row-major A, column-major B, M <= %d and K %% 8 == 0",
-                  SKINNY_MAX_M);
+        set_error("skinny rung needs a 16-bit float type, row-major A, column-major B, M <= %d and K %% %d == 0",
+                  SKINNY_MAX_M, SKINNY_K_STEP);
         return GZ_ERR_UNSUPPORTED;
       }
       if (variant > 1) { set_error("skinny rung has a single variant"); return GZ_ERR_UNSUPPORTED; }

@@ -125,7 +125,7 @@ __device__ inline float load_as_float(const void* p, int64_t i, int dtype) {
 }
 
 __global__ void __launch_bounds__(256) compare_kernel(const void* out, const void* ref, int64_t count, int dtype,
-                                                      float thr, unsigned long long* ndiff) {
+                                                      float thr, float rel, unsigned long long* ndiff) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   unsigned long long local = 0;
@@ -133,10 +133,11 @@ __global__ void __launch_bounds__(256) compare_kernel(const void* out, const voi
     bool diff;
     if (dtype == 4) {
       const int32_t a = static_cast<const int32_t*>(out)[i], b = static_cast<const int32_t*>(ref)[i];
-      diff = thr == 0.0f ? (a != b) : (fabs((double)a - (double)b) > (double)thr);
+      diff = (thr == 0.0f && rel == 0.0f) ? (a != b)
+                                          : (fabs((double)a - (double)b) > (double)thr + (double)rel * fabs((double)b));
     } else {
       const float a = load_as_float(out, i, dtype), b = load_as_float(ref, i, dtype);
-      diff = thr == 0.0f ? (a != b) : !(fabsf(a - b) <= thr);
+      diff = (thr == 0.0f && rel == 0.0f) ? (a != b) : !(fabsf(a - b) <= thr + rel * fabsf(b));
     }
     local += diff ? 1u : 0u;
   }
@@ -164,9 +165,9 @@ int gz_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t
   return GZ_OK;
 }
 
-int gz_compare(const void* out, const void* ref, int64_t count, int dtype, float abs_threshold,
-               int64_t* num_different, gz_stream stream) {
-  if (count < 0 || dtype < 0 || dtype > 4 || abs_threshold < 0.0f) {
+int gz_compare_rel(const void* out, const void* ref, int64_t count, int dtype, float abs_threshold,
+                   float rel_threshold, int64_t* num_different, gz_stream stream) {
+  if (count < 0 || dtype < 0 || dtype > 4 || !(abs_threshold >= 0.0f) || !(rel_threshold >= 0.0f)) {
     set_error("gz_compare: bad argument (count=%lld dtype=%d)", (long long)count, dtype);
     return GZ_ERR_BAD_ARG;
   }
@@ -185,7 +186,7 @@ int gz_compare(const void* out, const void* ref, int64_t count, int dtype, float
     }
     const int64_t blocks = (count + 255) / 256;
     const dim3 grid((unsigned)(blocks < 16384 ? blocks : 16384)), block(256);
-    hipLaunchKernelGGL(compare_kernel, grid, block, 0, s, out, ref, count, dtype, abs_threshold, d_count);
+    hipLaunchKernelGGL(compare_kernel, grid, block, 0, s, out, ref, count, dtype, abs_threshold, rel_threshold, d_count);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) { st = hip_fail(e, "compare launch"); break; }
     if (hipError_t e = hipMemcpyAsync(&h_count, d_count, sizeof(h_count), hipMemcpyDeviceToHost, s); e != hipSuccess) {
       st = hip_fail(e, "hipMemcpyAsync");
@@ -201,6 +202,11 @@ int gz_compare(const void* out, const void* ref, int64_t count, int dtype, float
     return GZ_ERR_MISMATCH;
   }
   return GZ_OK;
+}
+
+int gz_compare(const void* out, const void* ref, int64_t count, int dtype, float abs_threshold,
+               int64_t* num_different, gz_stream stream) {
+  return gz_compare_rel(out, ref, count, dtype, abs_threshold, 0.0f, num_different, stream);
 }
 
 }  // extern "C"

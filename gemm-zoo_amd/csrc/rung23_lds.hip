@@ -67,7 +67,9 @@ template <int TYPES, bool KC> struct SlabLoader {
 };
 
 template <int TYPES, bool A_KC, bool B_KC, int STAGES>
-__global__ void __launch_bounds__(LT_NT) lds_gemm_kernel(GemmArgs<TYPES> g) {
+// second launch bound: at least 4 waves per SIMD, i.e. at most 128 VGPRs -- without it the double-buffered
+// instantiation hoists every LDS read of a slab above the FMAs and ends up with one wave per SIMD
+__global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
   using T = Traits<TYPES>;
   using in_t = typename T::in_t;
   using acc_t = typename T::acc_t;
@@ -97,7 +99,7 @@ __global__ void __launch_bounds__(LT_NT) lds_gemm_kernel(GemmArgs<TYPES> g) {
   const int slabs = (K + LT_BK - 1) / LT_BK;
 
   auto compute = [&](const acc_t* as, const acc_t* bs) {
-#pragma unroll
+#pragma unroll 8
     for (int k = 0; k < LT_BK; k++) {
       const acc4_t a = *reinterpret_cast<const acc4_t*>(as + k * LT_PITCH + ty * 4);
       const acc4_t b = *reinterpret_cast<const acc4_t*>(bs + k * LT_PITCH + tx * 4);

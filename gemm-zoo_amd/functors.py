@@ -1,0 +1,136 @@
+"""Host-side mirror of gemm-zoo's kernel functors (``nvidia/kernel_functors/*.cuh``, ``intel/xe_gemm_*.hpp``).
+
+A functor is built for one problem size -- ``Kernel(m, n, k, props)`` resolves the launch plan the way the
+reference's constructors compute grid / block / shared memory and rejects what the rung cannot run -- and is then
+called as ``kernel(a, b, c, d, alpha, beta, stream)`` with device buffers (torch tensors or raw pointers); the
+launch is asynchronous on ``stream``.  ``functor(name, TIn, TOut, ...)`` plays the part of a template
+instantiation.  The C++ header ``include/gemm_zoo/kernel_functors.hpp`` is the same surface for C++ drivers.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from pathlib import Path
+
+from . import capi
+
+ROW, COL = capi.ROW_MAJOR, capi.COL_MAJOR
+
+# (TIn, TOut) -> type bundle, spelled as in the reference's drivers
+BUNDLES = {("s8", "s32"): capi.S8S8S32, ("bf16", "f32"): capi.BF16BF16F32, ("bf16", "bf16"): capi.BF16BF16BF16,
+           ("f16", "f16"): capi.F16F16F16}
+
+# functor name -> (rung, tile ints -> variant)
+_RUNGS = {
+    "naive_gemm": capi.RUNG_NAIVE,
+    "coalesced_gemm": capi.RUNG_COALESCED,
+    "generic_gemm": capi.RUNG_LDS_TILED,          # the any-shape fallback of nvidia/kernel_functors/generic_gemm.cuh
+    "smem_tiled_gemm": capi.RUNG_LDS_TILED,
+    "rmem_tiled_gemm": capi.RUNG_LDS_TILED,
+    "double_buffered_gemm": capi.RUNG_DOUBLE_BUFFERED,
+    "async_buffered_gemm": capi.RUNG_DOUBLE_BUFFERED,
+    "bf16_mma_gemm": capi.RUNG_MFMA,
+    "fp16_mma_gemm": capi.RUNG_MFMA,
+    "s8_mma_gemm": capi.RUNG_MFMA,
+    "gemm_s8_s8_s32_m8k16": capi.RUNG_AUTO,       # intel/xe_gemm_s8_s8_s32_m8k16.hpp:12
+    "gemm_bf16_bf16_f32_m8k16": capi.RUNG_AUTO,   # intel/xe_gemm_bf16_bf16_f32_m8k16.hpp:12
+    "gemm_bf16_bf16_bf16_m8k16": capi.RUNG_AUTO,  # intel/xe_gemm_bf16_bf16_bf16_m8k16.hpp:12
+    "auto_gemm": capi.RUNG_AUTO,
+    "skinny_gemm": capi.RUNG_SKINNY,
+}
+
+
+@dataclass
+class DeviceProps:
+    """The two fields of hipDeviceProp_t the launcher looks at."""
+    multiProcessorCount: int = 256
+    maxSharedMemoryPerMultiProcessor: int = 160 * 1024
+
+    @staticmethod
+    def current() -> "DeviceProps":
+        import torch
+
+        p = torch.cuda.get_device_properties(torch.cuda.current_device())
+        return DeviceProps(p.multi_processor_count, 160 * 1024)
+
+
+def _stream_ptr(stream) -> int:
+    if stream is None:
+        return 0
+    return stream if isinstance(stream, int) else stream.cuda_stream
+
+
+class KernelFunctor:
+    name = "auto_gemm"
+    types = capi.BF16BF16F32
+    layout_a = ROW
+    layout_b = ROW
+    rung = capi.RUNG_AUTO
+    variant = 0
+
+    def __init__(self, m: int, n: int, k: int, props: DeviceProps | None = None):
+        props = props or DeviceProps()
+        self.m, self.n, self.k = int(m), int(n), int(k)
+        # raises capi.GzError for shapes / layouts the rung cannot run (the reference asserts)
+        self.plan = capi.plan(self.types, self.m, self.n, self.k, self.layout_a, self.layout_b, self.rung,
+                              self.variant, props.multiProcessorCount, props.maxSharedMemoryPerMultiProcessor)
+
+    def __call__(self, a, b, c, d, alpha, beta, stream=None) -> None:
+        capi.gemm(self.types, a, b, c, d, self.m, self.n, self.k, self.layout_a, self.layout_b, alpha, beta,
+                  self.rung, self.variant, _stream_ptr(stream))
+
+
+def functor(name: str, tin: str, tout: str, *tile, layout_a: int = ROW, layout_b: int = ROW, variant: int = 0):
+    """``functor("bf16_mma_gemm", "bf16", "f32", 128, 128, 32)`` ~ ``bf16_mma_gemm<bf16_t, float, 128, 128, 32>``."""
+    if name not in _RUNGS:
+        raise KeyError(f"unknown kernel functor {name!r}")
+    if (tin, tout) not in BUNDLES:
+        raise KeyError(f"no type bundle for TIn={tin!r}, TOut={tout!r}")
+    rung = _RUNGS[name]
+    variant = int(variant)  # the reference's tile integers are a hint; `variant` pins a gfx950 tile configuration
+    return type(f"{name}<{tin},{tout}{''.join(',%d' % t for t in tile)}>", (KernelFunctor,),
+                dict(name=name, types=BUNDLES[(tin, tout)], layout_a=layout_a, layout_b=layout_b, rung=rung,
+                     variant=variant))
+
+
+class HipblasLtGemm:
+    """The vendor-library comparator (nvidia/kernel_functors/cublaslt_gemm.cuh:15-125); owns and frees its plan."""
+    _lib = None
+
+    @classmethod
+    def lib(cls):
+        if cls._lib is None:
+            path = Path(capi.LIB_PATH).with_name("libgemmzoo_hipblaslt.so")
+            if not path.exists():
+                raise ImportError(f"{path} is missing: build it with `python gemm-zoo_amd/build.py`")
+            lib = C.CDLL(str(path))
+            vp, i64, i32, f64 = C.c_void_p, C.c_int64, C.c_int, C.c_double
+            lib.gz_hipblaslt_create.argtypes = [i32, i64, i64, i64, i32, i32, C.POINTER(vp)]
+            lib.gz_hipblaslt_run.argtypes = [vp, vp, vp, vp, vp, f64, f64, vp]
+            lib.gz_hipblaslt_destroy.argtypes = [vp]
+            lib.gz_hipblaslt_last_error.restype = C.c_char_p
+            cls._lib = lib
+        return cls._lib
+
+    def __init__(self, types: int, m: int, n: int, k: int, layout_a: int = ROW, layout_b: int = ROW):
+        self._plan = C.c_void_p()
+        st = self.lib().gz_hipblaslt_create(types, m, n, k, layout_a, layout_b, C.byref(self._plan))
+        if st != capi.OK:
+            raise capi.GzError(st, self.lib().gz_hipblaslt_last_error().decode())
+
+    def __call__(self, a, b, c, d, alpha, beta, stream=None) -> None:
+        st = self.lib().gz_hipblaslt_run(self._plan, capi._ptr(a), capi._ptr(b), capi._ptr(c), capi._ptr(d),
+                                         float(alpha), float(beta), _stream_ptr(stream))
+        if st != capi.OK:
+            raise capi.GzError(st, self.lib().gz_hipblaslt_last_error().decode())
+
+    def close(self) -> None:
+        if self._plan:
+            self.lib().gz_hipblaslt_destroy(self._plan)
+            self._plan = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -143,6 +143,12 @@ int gz_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t
 int gz_compare(const void* out, const void* ref, int64_t count, int dtype,
                float abs_threshold, int64_t* num_different, gz_stream stream);
 
+/* As gz_compare with a mixed bound: an element differs when |out - ref| > abs_threshold + rel_threshold * |ref|
+ * (both zero: exact equality).  For 16-bit outputs, whose rounding step grows with the value, an absolute
+ * bound alone (nvidia/utils/compare.cuh:19 uses 0.5) is either too loose or too tight. */
+int gz_compare_rel(const void* out, const void* ref, int64_t count, int dtype, float abs_threshold,
+                   float rel_threshold, int64_t* num_different, gz_stream stream);
+
 const char* gz_last_error(void);
 int gz_version(void);
 

@@ -40,6 +40,8 @@ def test_compare_exact_and_threshold(G):
     b[17] += 0.25; b[99999] -= 1.0
     assert G.capi.compare(a, b, n, O.DT_F32, 0.0) == 2          # exact: intel/test/utils.hpp:57
     assert G.capi.compare(a, b, n, O.DT_F32, 0.5) == 1          # abs threshold: nvidia/utils/compare.cuh:19
+    assert G.capi.compare(a, b, n, O.DT_F32, 0.0, rel_threshold=1e-4) == 1   # 0.25 at 17 is out, 1.0 at 99999 is in
+    assert G.capi.compare(a, b, n, O.DT_F32, 0.2, rel_threshold=1e-2) == 0
     st = G.capi.lib.gz_compare(a.data_ptr(), b.data_ptr(), n, O.DT_F32, 0.0, None, None)
     assert st == G.capi.ERR_MISMATCH and "verification failed" in G.capi.last_error()
     i = torch.arange(n, dtype=torch.int32, device="cuda"); j = i.clone(); j[5] += 1
