@@ -37,6 +37,9 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="skip the s8 8192^3 and skinny side measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one plain 256 MiB device copy (known traffic) so that a counter run of this "
+                         "command holds the scale for FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -120,6 +123,14 @@ def main() -> int:
         return {"wall_ms": wall_ms, "kernel_ms_mean": sum(ev) / len(ev), "kernel_ms_median": ev[len(ev) // 2],
                 "problem_bytes": problem_bytes, "sets": p}
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        capi.fill(src, 256 << 20, capi.DT_INT8, capi.FILL_INT8_UNIFORM, 1.0, 1, sptr)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---------------- headline: bf16 4096^3, A row-major, B column-major, f32 out ----------------
     M = N = K = 4096
     flops = 2.0 * M * N * K
@@ -145,7 +156,7 @@ def main() -> int:
                                "alpha=1 beta=0, fp32 accumulate",
                    "rotating_input_sets": r["sets"], "plan": plan},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": measured_traffic(),
                      "kernel_ms_mean": round(r["kernel_ms_mean"], 5), "kernel_ms_median": round(r["kernel_ms_median"], 5)},
     }
 
@@ -172,6 +183,18 @@ def main() -> int:
 
     print(json.dumps(out))
     return 0
+
+
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a
+    plain copy of known size); the figures and the commands that produced them are in profiles/."""
+    f = ROOT / "profiles" / "mfma_bf16_4096_traffic.json"
+    if not f.exists():
+        return None
+    try:
+        return json.loads(f.read_text())["hbm_bytes_per_launch"]
+    except Exception:
+        return None
 
 
 def cpu_baseline(M, N, K, target_seconds):
