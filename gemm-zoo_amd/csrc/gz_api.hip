@@ -247,7 +247,7 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       plan->variant = 1;
       plan->tile_m = c.mb; plan->tile_n = c.cols_per_wg; plan->tile_k = c.k_per_split;
       plan->wave_m = c.mb; plan->wave_n = c.cols_per_wave;
-      plan->threads = c.threads; plan->split_k = c.split_k;
+      plan->threads = c.threads; plan->split_k = c.split_k; plan->lds_bytes = c.lds_bytes;
       plan->grid = (int64_t)c.grid_n * c.split_k;
       return GZ_OK;
     }

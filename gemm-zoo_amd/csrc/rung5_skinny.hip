@@ -1,18 +1,32 @@
-// Rung 5: weight-streaming kernel for decode-shaped problems (M <= 32).
+// Rung 5: weight-streaming kernels for decode-shaped problems (M <= 32).
 //
-// The weight matrix B (N x K, K contiguous) is read exactly once, straight from
-// global memory into MFMA operand registers; nothing about it is staged in LDS
-// because no element is reused by another wave.  One wavefront owns 16 output
-// columns and walks the whole of K in super-steps of 64 elements: the four
-// 16-lane groups of the wave each read 32 contiguous bytes of a weight row, so
-// every super-step consumes whole 128-byte lines.  Activations (M x K, at most
-// 256 KiB) are re-read by every wave and are served by L2.  Loads are issued
-// PF super-steps ahead of their use to keep enough bytes in flight to cover
-// HBM latency.
+// The weight matrix B (N x K, K contiguous) is read exactly once and nothing about it is reused by another
+// wave, so the kernel is a streaming read of B with a little matrix-core work attached.  What decides its
+// speed on MI355X (measured):
+//   * a compute unit sustains only a limited number of outstanding memory requests, so the chip's bandwidth is
+//     reached only when every compute unit streams its equal share: the columns are dealt out in equal
+//     groups of at most 32, 4-column granular, one or two groups per compute unit (cols_per_wg);
+//   * rows of B are a multiple of 4 KiB apart for the usual K, so work-groups that walk K in step all hit the
+//     same L2 / memory channel at the same moment: every work-group starts at a different K chunk (rot);
+//   * each byte is used once: the copies carry the non-temporal hint.
 //
-// v_mfma_f32_16x16x32_{bf16,f16}: the weight fragment is the first operand, so
-// a lane ends with 4 consecutive columns of one output row (64-bit stores).
+// skinny_dtl_kernel (K % 128 == 0): a work-group of KS waves owns up to 32 columns; its waves take the
+// 128-element K chunks round-robin.  A wave moves its chunk of the 32 rows (8 KiB) from global memory straight
+// into a private LDS ring with global_load_lds_dwordx4 -- every instruction moves four 256-byte row pieces --
+// and reads the MFMA fragments back with ds_read_b128; the 16-byte pieces of a row are XOR-swizzled with the
+// row number on the way in, so the reads are bank-conflict free.  There is no barrier in the main loop and
+// S stages are in flight per wave; the waits are hand-counted (the compiler does not see LDS-DMA).  The K
+// partial sums of the KS waves meet in LDS at the end.  Activations (at most 32 rows) come from L2 into
+// registers with the same depth.
+//
+// skinny_reg_kernel (K % 64 == 0 only): the earlier design, B straight into MFMA operand registers.
+//
+// v_mfma_f32_16x16x32_{bf16,f16}: the weight fragment is the first operand, so a lane ends with 4 consecutive
+// columns of one output row (64-bit stores).
 #include "gz_common.hpp"
+#include <type_traits>
+#include <utility>
+
 #include "gz_skinny_cfg.hpp"
 
 namespace gz {
@@ -33,7 +47,7 @@ __device__ inline sk_f32x4_t mfma16(sk_u32x4_t first, sk_u32x4_t second, sk_f32x
 }
 
 template <int TYPES, int MBLK, int WAVES, int PF>
-__global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(GemmArgs<TYPES> g) {
+__global__ void __launch_bounds__(WAVES * 64) skinny_reg_kernel(GemmArgs<TYPES> g) {
   using T = Traits<TYPES>;
   using in_t = typename T::in_t;
   using out_t = typename T::out_t;
@@ -119,6 +133,214 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(GemmArgs<TYPES>
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------
+// Direct-to-LDS streaming kernel
+// ---------------------------------------------------------------------------------------------------------
+template <class F, int... I> __device__ __forceinline__ void sk_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F> __device__ __forceinline__ void sk_for(F&& f) {
+  sk_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+template <int OFF> __device__ __forceinline__ void sk_ds_read16(sk_u32x4_t& dst, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
+}
+__device__ __forceinline__ void sk_set_m0(uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory");
+}
+// 64 lanes x 16 bytes, global (sbase + voff + OFF) -> LDS (M0 + OFF + 16 * lane); lanes outside `mask` move nothing
+// but the instruction still takes its place in the vmcnt order
+template <int OFF> __device__ __forceinline__ void sk_copy16(uint32_t voff, const void* sbase_minus_off, uint64_t mask) {
+  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
+  asm volatile("s_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2 nt\n\ts_mov_b64 exec, -1"
+               :
+               : "v"(voff), "s"(sbase_minus_off), "i"(OFF), "s"(mask)
+               : "memory");
+}
+template <int OFF> __device__ __forceinline__ void sk_load16(sk_u32x4_t& dst, uint32_t voff, const void* sbase) {
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=&v"(dst) : "v"(voff), "s"(sbase), "i"(OFF) : "memory");
+}
+template <int N> __device__ __forceinline__ void sk_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "i"(N) : "memory"); }
+__device__ __forceinline__ void sk_wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
+// orders later uses of a register after the asm statements that precede this one
+__device__ __forceinline__ void sk_touch(sk_u32x4_t& v) { asm volatile("" : "+v"(v)); }
+
+template <int TYPES, int MBLK, int KS, int S>
+__global__ void __launch_bounds__(KS * 64) skinny_dtl_kernel(GemmArgs<TYPES> g, int cols_per_wg) {
+  using T = Traits<TYPES>;
+  using out_t = typename T::out_t;
+  extern __shared__ __attribute__((aligned(1024))) char sk_lds[];
+  constexpr int CB = 2;                          // 16-column MFMA blocks per work-group
+  constexpr int NCP = CB * 4;                    // 1 KiB copies per stage (4 rows x 256 bytes each)
+  constexpr int STAGE = SKINNY_DTL_STAGE_BYTES;  // 32 rows x 256 bytes
+  constexpr int PER = NCP + 4 * MBLK;            // vector-memory instructions per stage
+  constexpr int NA = MBLK * CB;
+  static_assert((S - 1) * PER < 64, "vmcnt is a 6-bit counter");
+  const uint32_t lds_base = (uint32_t)(uintptr_t)sk_lds;
+  const int lane = threadIdx.x & 63;
+  const int ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n_base = blockIdx.x * cols_per_wg;
+  const int K = g.K, N = g.N, M = g.M;
+  const uint32_t ring = lds_base + ks * (S * STAGE);
+  const size_t rowb = (size_t)K * 2;
+
+  // copy j moves rows 4j .. 4j+3 of the group: 16 lanes per row; the lane that fills position p of the LDS row
+  // fetches piece p ^ (row & 15) of the 256-byte chunk.  (n - n_base) * rowb < 2 * N * K < 2^32.
+  uint32_t voff[NCP];
+#pragma unroll
+  for (int j = 0; j < NCP; j++) {
+    const int row = 4 * j + (lane >> 4), p = lane & 15;
+    const int n = min(n_base + row, N - 1);
+    voff[j] = (uint32_t)((size_t)(n - n_base) * rowb) + (uint32_t)((p ^ (row & 15)) * 16);
+  }
+  const char* sb = reinterpret_cast<const char*>(g.B) + (size_t)n_base * rowb;
+  const int r16 = lane & 15, grp = lane >> 4;
+  uint32_t a_voff[MBLK];
+#pragma unroll
+  for (int mb = 0; mb < MBLK; mb++) a_voff[mb] = (uint32_t)((size_t)min(mb * 16 + r16, M - 1) * rowb) + grp * 16;
+  const char* sa = reinterpret_cast<const char*>(g.A);
+  // fragment of MFMA step t: row r16 of a column block, K piece 4t + grp
+  uint32_t b_addr[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) b_addr[t] = ring + r16 * 256 + (((t * 4 + grp) ^ r16) * 16);
+
+  sk_f32x4_t acc[MBLK][CB];
+#pragma unroll
+  for (int mb = 0; mb < MBLK; mb++)
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) acc[mb][cb] = sk_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  sk_u32x4_t aq[S][MBLK][4];
+
+  const int chunks = K / SKINNY_DTL_K_STEP;
+  const int mine = (chunks - ks + KS - 1) / KS;          // this wave's chunks: ks, ks + KS, ... (before rotation)
+  const int rot = (int)(blockIdx.x % (unsigned)chunks);
+
+  auto chunk_byte = [&](int i) {
+    int c = i * KS + ks + rot;
+    if (c >= chunks) c -= chunks;
+    return (size_t)c * 256;
+  };
+  auto issue_copies = [&](auto slot_c, int i) {
+    constexpr int SL = decltype(slot_c)::value;
+    const size_t kbyte = chunk_byte(i);
+    sk_for<CB>([&](auto q_c) {
+      constexpr int Q = decltype(q_c)::value;  // four copies share one M0
+      sk_set_m0(ring + SL * STAGE + Q * 4096 + 2048);
+      sk_for<4>([&](auto j_c) {
+        constexpr int J = decltype(j_c)::value;
+        // cols_per_wg is a multiple of 4: a copy moves four whole rows or nothing (mask as a scalar register pair)
+        const uint32_t on = (uint32_t)__builtin_amdgcn_readfirstlane(4 * (Q * 4 + J) < cols_per_wg ? -1 : 0);
+        sk_copy16<(J - 2) * 1024>(voff[Q * 4 + J], sb + kbyte - (J - 2) * 1024, ((uint64_t)on << 32) | on);
+      });
+    });
+  };
+  auto issue_a = [&](auto slot_c, int i) {
+    constexpr int SL = decltype(slot_c)::value;
+    const size_t kbyte = chunk_byte(i);
+    sk_for<MBLK>([&](auto mb_c) {
+      constexpr int MB = decltype(mb_c)::value;
+      sk_for<4>([&](auto t_c) {
+        constexpr int TT = decltype(t_c)::value;
+        sk_load16<TT * 64>(aq[SL][MB][TT], a_voff[MB], sa + kbyte);
+      });
+    });
+  };
+
+  sk_for<S>([&](auto sl) {
+    if (decltype(sl)::value < mine) {
+      issue_copies(sl, decltype(sl)::value);
+      issue_a(sl, decltype(sl)::value);
+    }
+  });
+
+  for (int i0 = 0; i0 < mine; i0 += S) {
+    sk_for<S>([&](auto sl) {
+      constexpr int SL = decltype(sl)::value;
+      const int i = i0 + SL;
+      if (i < mine) {
+        // stage i has landed once at most the S - 1 younger stages are outstanding
+        if (i + S - 1 < mine) sk_wait_vm<(S - 1) * PER>();
+        else sk_wait_vm<0>();
+        sk_u32x4_t bf[CB][4];
+        sk_for<CB>([&](auto cb_c) {
+          constexpr int CBI = decltype(cb_c)::value;
+          sk_for<4>([&](auto t_c) {
+            constexpr int TT = decltype(t_c)::value;
+            sk_ds_read16<SL * STAGE + CBI * 4096>(bf[CBI][TT], b_addr[TT]);
+          });
+        });
+        sk_wait_lgkm0();
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+          for (int t = 0; t < 4; t++) sk_touch(bf[cb][t]);
+#pragma unroll
+        for (int mb = 0; mb < MBLK; mb++)
+#pragma unroll
+          for (int t = 0; t < 4; t++) sk_touch(aq[SL][mb][t]);
+        const bool more = i + S < mine;
+        if (more) issue_copies(sl, i + S);  // the fragments are in registers: the stage buffer is free
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int mb = 0; mb < MBLK; mb++)
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) acc[mb][cb] = mfma16<TYPES>(bf[cb][t], aq[SL][mb][t], acc[mb][cb]);
+        if (more) issue_a(sl, i + S);
+      }
+    });
+  }
+
+  // every wave has waited for all of its copies (the last stages wait with vmcnt(0)): the rings can be reused
+  float* red = reinterpret_cast<float*>(sk_lds);
+  if constexpr (KS > 1) {
+    __syncthreads();
+#pragma unroll
+    for (int mb = 0; mb < MBLK; mb++)
+#pragma unroll
+      for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) red[((ks * NA + mb * CB + cb) * 4 + e) * 64 + lane] = acc[mb][cb][e];
+    __syncthreads();
+    if (ks != 0) return;
+#pragma unroll
+    for (int w = 1; w < KS; w++)
+#pragma unroll
+      for (int mb = 0; mb < MBLK; mb++)
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[mb][cb][e] += red[((w * NA + mb * CB + cb) * 4 + e) * 64 + lane];
+  }
+
+  // acc[mb][cb][v] = D(16 mb + r16, n_base + 16 cb + 4 grp + v)
+  const int n_end = min(n_base + cols_per_wg, N);
+  const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
+                      (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
+#pragma unroll
+  for (int mb = 0; mb < MBLK; mb++) {
+    const int m = mb * 16 + r16;
+    if (m >= M) continue;
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+      const int n = n_base + cb * 16 + 4 * grp;
+      const size_t o = (size_t)m * N + n;
+      if (vec_ok && n + 3 < n_end) {
+        out_t cv[4] = {0, 0, 0, 0}, dv[4];
+        if (g.beta != 0) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+#pragma unroll
+        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[mb][cb][e], g.alpha, g.beta, &cv[e]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(acc[mb][cb][e], g.alpha, g.beta, g.C + o + e);
+      }
+    }
+  }
+}
+
 template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
   if constexpr (TYPES == GZ_S8S8S32) {
     (void)g; (void)variant; (void)s;
@@ -140,8 +362,20 @@ template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hi
     }
     const SkinnyCfg c = skinny_resolve(g.M, g.N, g.K, 256);
     const dim3 grid((unsigned)c.grid_n), block((unsigned)c.threads);
-    if (c.mb == 16) hipLaunchKernelGGL((skinny_gemm_kernel<TYPES, 1, 2, 4>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((skinny_gemm_kernel<TYPES, 2, 2, 4>), grid, block, 0, s, g);
+    if (c.dtl) {
+      constexpr int KS = SKINNY_DTL_WAVES, S = SKINNY_DTL_STAGES;
+      auto k1 = skinny_dtl_kernel<TYPES, 1, KS, S>;
+      auto k2 = skinny_dtl_kernel<TYPES, 2, KS, S>;
+      auto kern = c.mb == 16 ? k1 : k2;
+      // more than 64 KiB of dynamic LDS needs the opt-in; harmless below
+      GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     c.lds_bytes));
+      hipLaunchKernelGGL(kern, grid, block, c.lds_bytes, s, g, c.cols_per_wg);
+    } else if (c.mb == 16) {
+      hipLaunchKernelGGL((skinny_reg_kernel<TYPES, 1, 2, 4>), grid, block, 0, s, g);
+    } else {
+      hipLaunchKernelGGL((skinny_reg_kernel<TYPES, 2, 2, 4>), grid, block, 0, s, g);
+    }
     GZ_HIP_TRY(hipGetLastError());
     return GZ_OK;
   }
