@@ -61,7 +61,7 @@ static int check_problem(int types, int64_t M, int64_t N, int64_t K, int layoutA
 
 static int resolve_rung(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung) {
   if (rung != GZ_RUNG_AUTO) return rung;
-  if (skinny_supported(types, (int)M, (int)N, (int)K, layoutA, layoutB)) return GZ_RUNG_SKINNY;
+  if (skinny_preferred(types, (int)M, (int)N, (int)K, layoutA, layoutB, 0)) return GZ_RUNG_SKINNY;
   return GZ_RUNG_MFMA;
 }
 
@@ -245,8 +245,9 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       if (variant > 1) { set_error("skinny rung has a single variant"); return GZ_ERR_UNSUPPORTED; }
       SkinnyCfg c = skinny_resolve(m, n, k, num_cus);
       plan->variant = 1;
-      plan->tile_m = c.mb; plan->tile_n = c.cols_per_wg; plan->tile_k = c.k_per_split;
-      plan->wave_m = c.mb; plan->wave_n = c.cols_per_wave;
+      plan->tile_m = c.mb; plan->tile_n = c.cols_per_wg;
+      plan->tile_k = c.kind == SKINNY_KIND_TILE ? STREAM_TILE_K_STEP : c.kind == SKINNY_KIND_DTL ? SKINNY_DTL_K_STEP : SKINNY_K_STEP;
+      plan->wave_m = c.kind == SKINNY_KIND_TILE ? 32 : c.mb; plan->wave_n = c.cols_per_wave;
       plan->threads = c.threads; plan->split_k = c.split_k; plan->lds_bytes = c.lds_bytes;
       plan->grid = (int64_t)c.grid_n * c.split_k;
       return GZ_OK;

@@ -6,7 +6,8 @@
 
 namespace gz {
 
-constexpr int SKINNY_MAX_M = 32;       // rows of activations the streaming kernel keeps per wave
+constexpr int SKINNY_MAX_M = 128;      // most rows of activations the streaming kernels take
+constexpr int SKINNY_REG_MAX_M = 16;   // above: activations are shared through LDS (stream_tile_kernel)
 constexpr int SKINNY_COLS_PER_WAVE = 16;
 constexpr int SKINNY_K_STEP = 64;      // elements of K consumed per super-step (128 bytes per weight row)
 // direct-to-LDS kernel: 128-element K chunks, 32 rows x 256 bytes per stage, waves per work-group, stages per wave
@@ -14,9 +15,18 @@ constexpr int SKINNY_DTL_K_STEP = 128;
 constexpr int SKINNY_DTL_STAGE_BYTES = 8192;
 constexpr int SKINNY_DTL_WAVES = 4;
 constexpr int SKINNY_DTL_STAGES = 2;
+// producer / consumer tile kernel: 64 K elements (128-byte rows) per stage, at most 64 columns per work-group,
+// four consumer and four producer waves, ring depth by number of 32-row blocks of A
+constexpr int STREAM_TILE_K_STEP = 64;
+constexpr int STREAM_TILE_ROW_BYTES = 128;
+constexpr int STREAM_TILE_COLS = 64;
+constexpr int STREAM_TILE_THREADS = 512;
+constexpr int STREAM_TILE_STAGES_1 = 8, STREAM_TILE_STAGES_2 = 4, STREAM_TILE_STAGES_4 = 4;
+
+enum { SKINNY_KIND_REG = 0, SKINNY_KIND_DTL = 1, SKINNY_KIND_TILE = 2 };
 
 struct SkinnyCfg {
-  int mb;             // rows padded to a multiple of 16
+  int mb;             // rows of A the kernel instance covers: 16, 32, 64 or 128
   int cols_per_wave;  // 16
   int waves;          // wavefronts per work-group
   int cols_per_wg;
@@ -24,7 +34,7 @@ struct SkinnyCfg {
   int grid_n;         // work-groups along N
   int split_k;        // K slices (partial sums reduced by a second kernel when > 1)
   int k_per_split;
-  int dtl;            // 1: direct-to-LDS kernel (K % 128 == 0), 0: register-streaming kernel
+  int kind;           // SKINNY_KIND_*
   int lds_bytes;
 };
 
@@ -37,30 +47,48 @@ inline bool skinny_supported(int types, int M, int N, int K, int layoutA, int la
   return K % SKINNY_K_STEP == 0;
 }
 
+// What the launcher's own choice sends here: always the register-resident cases; the LDS-shared tile kernel only
+// while the tiled MFMA rung could not give every compute unit a 128 x 128 tile of its own.
+inline bool skinny_preferred(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus) {
+  if (!skinny_supported(types, M, N, K, layoutA, layoutB)) return false;
+  if (num_cus <= 0) num_cus = 256;
+  return M <= 32 || (long long)((N + 127) / 128) <= num_cus;
+}
+
+// equal column groups, one or more per compute unit, at most max_cols columns and a multiple of 4 each
+inline int skinny_balanced_cols(int N, int num_cus, int max_cols) {
+  if (num_cus <= 0) num_cus = 256;
+  for (int w = 1; w <= 1024; w++) {
+    const long long slots = (long long)num_cus * w;
+    int per = (int)((N + slots - 1) / slots);
+    per = (per + 3) / 4 * 4;
+    if (per <= max_cols) return per;
+  }
+  return max_cols;
+}
+
 inline SkinnyCfg skinny_resolve(int M, int N, int K, int num_cus) {
   SkinnyCfg c;
-  c.mb = M <= 16 ? 16 : 32;
   c.split_k = 1;
   c.k_per_split = K;
-  c.dtl = K % SKINNY_DTL_K_STEP == 0;
-  if (c.dtl) {
-    // equal column groups, one or more per compute unit, at most 32 columns and a multiple of 4 each
-    if (num_cus <= 0) num_cus = 256;
-    int cols = 32;
-    for (int w = 1; w <= 64; w++) {
-      const long long slots = (long long)num_cus * w;
-      int per = (int)((N + slots - 1) / slots);
-      per = (per + 3) / 4 * 4;
-      if (per <= 32) {
-        cols = per;
-        break;
-      }
-    }
-    c.cols_per_wave = cols;          // every wave of the work-group works on all of its columns (K is split)
+  if (M > SKINNY_REG_MAX_M) {
+    c.kind = SKINNY_KIND_TILE;
+    c.mb = M <= 32 ? 32 : M <= 64 ? 64 : 128;
+    const int stages = c.mb == 32 ? STREAM_TILE_STAGES_1 : c.mb == 64 ? STREAM_TILE_STAGES_2 : STREAM_TILE_STAGES_4;
+    c.cols_per_wg = skinny_balanced_cols(N, num_cus, STREAM_TILE_COLS);
+    c.cols_per_wave = 32;
+    c.waves = STREAM_TILE_THREADS / 64;
+    c.lds_bytes = stages * (c.mb + STREAM_TILE_COLS) * STREAM_TILE_ROW_BYTES;
+  } else if (K % SKINNY_DTL_K_STEP == 0) {
+    c.kind = SKINNY_KIND_DTL;
+    c.mb = 16;
+    c.cols_per_wg = skinny_balanced_cols(N, num_cus, 32);
+    c.cols_per_wave = c.cols_per_wg;  // every wave of the work-group works on all of its columns (K is split)
     c.waves = SKINNY_DTL_WAVES;
-    c.cols_per_wg = cols;
     c.lds_bytes = SKINNY_DTL_WAVES * SKINNY_DTL_STAGES * SKINNY_DTL_STAGE_BYTES;
   } else {
+    c.kind = SKINNY_KIND_REG;
+    c.mb = 16;
     c.cols_per_wave = SKINNY_COLS_PER_WAVE;
     c.waves = 2;
     c.cols_per_wg = c.cols_per_wave * c.waves;

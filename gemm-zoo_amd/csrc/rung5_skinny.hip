@@ -1,4 +1,4 @@
-// Rung 5: weight-streaming kernels for decode-shaped problems (M <= 32).
+// Rung 5: weight-streaming kernels for decode-shaped problems (M <= 128).
 //
 // The weight matrix B (N x K, K contiguous) is read exactly once and nothing about it is reused by another
 // wave, so the kernel is a streaming read of B with a little matrix-core work attached.  What decides its
@@ -10,16 +10,24 @@
 //     same L2 / memory channel at the same moment: every work-group starts at a different K chunk (rot);
 //   * each byte is used once: the copies carry the non-temporal hint.
 //
-// skinny_dtl_kernel (K % 128 == 0): a work-group of KS waves owns up to 32 columns; its waves take the
+// skinny_dtl_kernel (M <= 16, K % 128 == 0): a work-group of KS waves owns up to 32 columns; its waves take the
 // 128-element K chunks round-robin.  A wave moves its chunk of the 32 rows (8 KiB) from global memory straight
 // into a private LDS ring with global_load_lds_dwordx4 -- every instruction moves four 256-byte row pieces --
 // and reads the MFMA fragments back with ds_read_b128; the 16-byte pieces of a row are XOR-swizzled with the
 // row number on the way in, so the reads are bank-conflict free.  There is no barrier in the main loop and
 // S stages are in flight per wave; the waits are hand-counted (the compiler does not see LDS-DMA).  The K
-// partial sums of the KS waves meet in LDS at the end.  Activations (at most 32 rows) come from L2 into
+// partial sums of the KS waves meet in LDS at the end.  Activations (at most 16 rows) come from L2 into
 // registers with the same depth.
 //
-// skinny_reg_kernel (K % 64 == 0 only): the earlier design, B straight into MFMA operand registers.
+// skinny_reg_kernel (M <= 16, K % 64 == 0 only): the earlier design, B straight into MFMA operand registers.
+//
+// stream_tile_kernel (16 < M <= 128, K % 64 == 0): here the activations no longer fit a wave's registers and every
+// compute unit needs all of them, so they are shared through LDS.  One work-group per compute unit owns up to 64
+// columns.  Four producer waves move stage after stage (64 K elements: A rows and B rows, 128 bytes each, swizzled)
+// into a ring with direct-to-LDS copies; four consumer waves read the fragments and run v_mfma_f32_32x32x16.
+// Splitting the roles matters: a copy instruction occupies its wave for about 55 cycles however many lanes it
+// moves, and with one wave per SIMD doing both jobs the copy issue, the LDS reads and the MFMAs of a stage ran
+// back to back.  One barrier per stage says both "stage i has landed" and "stage i - 1 may be overwritten".
 //
 // v_mfma_f32_16x16x32_{bf16,f16}: the weight fragment is the first operand, so a lane ends with 4 consecutive
 // columns of one output row (64-bit stores).
@@ -35,6 +43,7 @@ typedef __bf16 sk_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 sk_f16x8_t __attribute__((ext_vector_type(8)));
 typedef float sk_f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t sk_u32x4_t __attribute__((ext_vector_type(4)));
+typedef float sk_f32x16_t __attribute__((ext_vector_type(16)));
 
 template <int TYPES>
 __device__ inline sk_f32x4_t mfma16(sk_u32x4_t first, sk_u32x4_t second, sk_f32x4_t acc) {
@@ -43,6 +52,16 @@ __device__ inline sk_f32x4_t mfma16(sk_u32x4_t first, sk_u32x4_t second, sk_f32x
                                                   __builtin_bit_cast(sk_f16x8_t, second), acc, 0, 0, 0);
   else
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8_t, first),
+                                                   __builtin_bit_cast(sk_bf16x8_t, second), acc, 0, 0, 0);
+}
+
+template <int TYPES>
+__device__ inline sk_f32x16_t mfma32x16(sk_u32x4_t first, sk_u32x4_t second, sk_f32x16_t acc) {
+  if constexpr (TYPES == GZ_F16F16F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(sk_f16x8_t, first),
+                                                  __builtin_bit_cast(sk_f16x8_t, second), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(sk_bf16x8_t, first),
                                                    __builtin_bit_cast(sk_bf16x8_t, second), acc, 0, 0, 0);
 }
 
@@ -154,6 +173,15 @@ __device__ __forceinline__ void sk_set_m0(uint32_t lds_addr) {
 template <int OFF> __device__ __forceinline__ void sk_copy16(uint32_t voff, const void* sbase_minus_off, uint64_t mask) {
   static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
   asm volatile("s_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2 nt\n\ts_mov_b64 exec, -1"
+               :
+               : "v"(voff), "s"(sbase_minus_off), "i"(OFF), "s"(mask)
+               : "memory");
+}
+// the same without the non-temporal hint (activations are re-read by every compute unit: keep them in L2)
+template <int OFF>
+__device__ __forceinline__ void sk_copy16_keep(uint32_t voff, const void* sbase_minus_off, uint64_t mask) {
+  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
+  asm volatile("s_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2\n\ts_mov_b64 exec, -1"
                :
                : "v"(voff), "s"(sbase_minus_off), "i"(OFF), "s"(mask)
                : "memory");
@@ -341,6 +369,174 @@ __global__ void __launch_bounds__(KS * 64) skinny_dtl_kernel(GemmArgs<TYPES> g, 
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------
+// Producer / consumer streaming tile kernel, 16 < M <= 128
+//   LDS ring: S stages of [A: 32 MB32 rows | B: 64 rows] x 128 bytes; piece p (16 bytes) of tile row r sits at
+//   position p ^ ((r >> 1) & 7), which makes the 32-row fragment reads bank-conflict free.
+//   Consumer wave w: column block w & 1; MB32 >= 2: row group w >> 1 (MB32 / 2 blocks of 32 rows), all four
+//   k-steps of a stage; MB32 == 1: the wave pairs split the k-steps and add their sums through LDS at the end.
+// ---------------------------------------------------------------------------------------------------------
+template <int TYPES, int MB32, int S>
+__global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmArgs<TYPES> g, int cols_per_wg) {
+  constexpr int NCW = 4;  // consumer waves; the four producer waves follow
+  using T = Traits<TYPES>;
+  using out_t = typename T::out_t;
+  extern __shared__ __attribute__((aligned(1024))) char sk_lds[];
+  constexpr int RB = STREAM_TILE_ROW_BYTES, B_BYTES = STREAM_TILE_COLS * RB, A_ROWS = MB32 * 32, A_BYTES = A_ROWS * RB, STAGE = A_BYTES + B_BYTES;
+  constexpr int NA = MB32, NB = 2, NCP = NA + NB;      // copies per producer wave and stage
+  // NCW consumer waves: 2 column blocks x NRG row groups x KSPLIT shares of the 4 MFMA k-steps of a stage
+  constexpr int NRG = MB32 >= 2 ? 2 : 1, NRB = MB32 / NRG, KSPLIT = NCW / (2 * NRG), NT = 4 / KSPLIT;
+  static_assert(KSPLIT >= 1 && NT >= 1, "");
+  static_assert(MB32 == 1 || MB32 == 2 || MB32 == 4, "");
+  static_assert((S - 2) * NCP < 64, "vmcnt");
+  const uint32_t lds_base = (uint32_t)(uintptr_t)sk_lds;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int K = g.K, N = g.N, M = g.M;
+  const int n_base = blockIdx.x * cols_per_wg;
+  const int n_end = min(n_base + cols_per_wg, N);
+  const size_t rowb = (size_t)K * 2;
+  const int nst = K / STREAM_TILE_K_STEP;
+  const int rot = (int)(blockIdx.x % (unsigned)nst);
+
+  if (wave >= NCW) {
+    // ---------------- producers: wave p moves A rows [8 NA p, 8 NA (p+1)) and B rows [16 p, 16 p + 16) of every stage ----------------
+    const int p = wave - NCW;
+    uint32_t voffA[NA], voffB[NB];
+    uint64_t maskB[NB];
+    const int row_in = lane >> 3, pos = lane & 7;
+#pragma unroll
+    for (int j = 0; j < NA; j++) {
+      const int row = (p * NA + j) * 8 + row_in;
+      voffA[j] = (uint32_t)((size_t)min(row, M - 1) * rowb) + (pos ^ ((row >> 1) & 7)) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+      const int row = (p * NB + j) * 8 + row_in;
+      const int n = min(n_base + row, N - 1);
+      voffB[j] = (uint32_t)((size_t)(n - n_base) * rowb) + (pos ^ ((row >> 1) & 7)) * 16;
+      maskB[j] = __builtin_amdgcn_ballot_w64(n_base + row < n_end);
+    }
+    const char* sA = reinterpret_cast<const char*>(g.A);
+    const char* sB = reinterpret_cast<const char*>(g.B) + (size_t)n_base * rowb;
+    int slot = 0;
+    auto issue = [&](int s) {   // a stage past the end: every copy masked off but still counted
+      const bool exists = s < nst;
+      int c = s + rot;
+      if (c >= nst) c -= nst;
+      if (!exists) c = 0;
+      const uint32_t dst = lds_base + (uint32_t)slot * STAGE;
+      slot = slot + 1 == S ? 0 : slot + 1;
+      sk_set_m0(dst + p * (NA * 1024) + 2048);
+      sk_for<NA>([&](auto j_c) {
+        constexpr int J = decltype(j_c)::value;
+        sk_copy16_keep<(J - 2) * 1024>(voffA[J], sA + (size_t)c * RB - (J - 2) * 1024, __builtin_amdgcn_ballot_w64(exists));
+      });
+      sk_set_m0(dst + A_BYTES + p * (NB * 1024) + 2048);
+      sk_for<NB>([&](auto j_c) {
+        constexpr int J = decltype(j_c)::value;
+        const uint64_t m = maskB[J] & __builtin_amdgcn_ballot_w64(exists);
+        sk_copy16<(J - 2) * 1024>(voffB[J], sB + (size_t)c * RB - (J - 2) * 1024, m);
+      });
+    };
+    for (int s = 0; s < S - 1; s++) issue(s);
+    for (int i = 0; i < nst; i++) {
+      sk_wait_vm<(S - 2) * NCP>();                 // stage i has landed
+      asm volatile("s_barrier" ::: "memory");     // consumers are done with stage i - 1
+      issue(i + S - 1);
+    }
+    sk_wait_vm<0>();
+    if constexpr (KSPLIT > 1) { __syncthreads(); __syncthreads(); }
+    return;
+  }
+
+  // ------------------------------------------- consumers: waves 0..3 -------------------------------------------
+  const int r32 = lane & 31, g2 = lane >> 5;
+  const int cbw = wave & 1, rb0 = ((wave >> 1) % NRG) * NRB;
+  const int kq = (wave >> 1) / NRG, t0 = kq * NT;
+  uint32_t b_addr[NT], a_addr[NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const int pp = ((2 * (t + t0) + g2) ^ ((r32 >> 1) & 7)) * 16;
+    a_addr[t] = lds_base + (rb0 * 32 + r32) * RB + pp;
+    b_addr[t] = lds_base + A_BYTES + (cbw * 32 + r32) * RB + pp;
+  }
+  sk_f32x16_t acc[NRB];
+#pragma unroll
+  for (int r = 0; r < NRB; r++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[r][e] = 0.f;
+
+  uint32_t so = 0;
+  for (int i = 0; i < nst; i++) {
+    asm volatile("s_barrier" ::: "memory");
+    sk_u32x4_t bf[NT], af[NRB][NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) sk_ds_read16<0>(bf[t], b_addr[t] + so);
+    sk_for<NRB>([&](auto r_c) {
+      constexpr int R = decltype(r_c)::value;
+#pragma unroll
+      for (int t = 0; t < NT; t++) sk_ds_read16<R * 32 * RB>(af[R][t], a_addr[t] + so);
+    });
+    so = so + STAGE == S * STAGE ? 0 : so + STAGE;
+    sk_wait_lgkm0();
+#pragma unroll
+    for (int t = 0; t < NT; t++) sk_touch(bf[t]);
+#pragma unroll
+    for (int r = 0; r < NRB; r++)
+#pragma unroll
+      for (int t = 0; t < NT; t++) sk_touch(af[r][t]);
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+      for (int r = 0; r < NRB; r++) acc[r] = mfma32x16<TYPES>(bf[t], af[r][t], acc[r]);
+  }
+  if constexpr (KSPLIT > 1) {
+    float* red = reinterpret_cast<float*>(sk_lds);
+    __syncthreads();   // every copy has landed and every fragment has been read: the rings are free
+    const int tile = wave % (2 * NRG);
+    if (kq > 0) {
+#pragma unroll
+      for (int r = 0; r < NRB; r++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) red[((((kq - 1) * 2 * NRG + tile) * NRB + r) * 16 + e) * 64 + lane] = acc[r][e];
+    }
+    __syncthreads();
+    if (kq > 0) return;
+#pragma unroll
+    for (int q = 1; q < KSPLIT; q++)
+#pragma unroll
+      for (int r = 0; r < NRB; r++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[r][e] += red[((((q - 1) * 2 * NRG + tile) * NRB + r) * 16 + e) * 64 + lane];
+  }
+
+  const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
+                      (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
+#pragma unroll
+  for (int r = 0; r < NRB; r++) {
+    const int m = (rb0 + r) * 32 + r32;
+    if (m >= M) continue;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int n = n_base + cbw * 32 + q * 8 + g2 * 4;
+      const size_t o = (size_t)m * N + n;
+      if (vec_ok && n + 3 < n_end) {
+        out_t cv[4] = {0, 0, 0, 0}, dv[4];
+        if (g.beta != 0) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+#pragma unroll
+        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[r][4 * q + e], g.alpha, g.beta, &cv[e]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(acc[r][4 * q + e], g.alpha, g.beta, g.C + o + e);
+      }
+    }
+  }
+}
+
 template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
   if constexpr (TYPES == GZ_S8S8S32) {
     (void)g; (void)variant; (void)s;
@@ -362,19 +558,23 @@ template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hi
     }
     const SkinnyCfg c = skinny_resolve(g.M, g.N, g.K, 256);
     const dim3 grid((unsigned)c.grid_n), block((unsigned)c.threads);
-    if (c.dtl) {
+    if (c.kind == SKINNY_KIND_TILE) {
+      auto k1 = stream_tile_kernel<TYPES, 1, STREAM_TILE_STAGES_1>;
+      auto k2 = stream_tile_kernel<TYPES, 2, STREAM_TILE_STAGES_2>;
+      auto k4 = stream_tile_kernel<TYPES, 4, STREAM_TILE_STAGES_4>;
+      auto kern = c.mb == 32 ? k1 : c.mb == 64 ? k2 : k4;
+      GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     c.lds_bytes));
+      hipLaunchKernelGGL(kern, grid, block, c.lds_bytes, s, g, c.cols_per_wg);
+    } else if (c.kind == SKINNY_KIND_DTL) {
       constexpr int KS = SKINNY_DTL_WAVES, S = SKINNY_DTL_STAGES;
-      auto k1 = skinny_dtl_kernel<TYPES, 1, KS, S>;
-      auto k2 = skinny_dtl_kernel<TYPES, 2, KS, S>;
-      auto kern = c.mb == 16 ? k1 : k2;
+      auto kern = skinny_dtl_kernel<TYPES, 1, KS, S>;
       // more than 64 KiB of dynamic LDS needs the opt-in; harmless below
       GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      c.lds_bytes));
       hipLaunchKernelGGL(kern, grid, block, c.lds_bytes, s, g, c.cols_per_wg);
-    } else if (c.mb == 16) {
-      hipLaunchKernelGGL((skinny_reg_kernel<TYPES, 1, 2, 4>), grid, block, 0, s, g);
     } else {
-      hipLaunchKernelGGL((skinny_reg_kernel<TYPES, 2, 2, 4>), grid, block, 0, s, g);
+      hipLaunchKernelGGL((skinny_reg_kernel<TYPES, 1, 2, 4>), grid, block, 0, s, g);
     }
     GZ_HIP_TRY(hipGetLastError());
     return GZ_OK;

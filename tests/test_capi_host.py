@@ -39,7 +39,7 @@ def test_version_and_names(capi):
     (dict(rung=4, variant=99), 2),
     (dict(rung=0, variant=1), 2),
     (dict(types=0, rung=5), 2),                 # no int8 streaming kernel
-    (dict(rung=5, m=64, layout_b=1), 2),        # M too large for the streaming kernel
+    (dict(rung=5, m=129, layout_b=1), 2),       # M too large for the streaming kernels
     (dict(rung=5, m=8, layout_b=0), 2),         # needs column-major weights
     (dict(rung=5, m=8, layout_b=1, k=100), 2),  # K not a whole number of super-steps
 ])
@@ -92,10 +92,19 @@ def test_plan_headline_configs(capi):
     assert p.grid == -(-4095 // p.tile_m) * -(-4097 // p.tile_n)
     assert p.vector_bytes_a == 2 and p.vector_bytes_b == 2
     # decode shapes go to the streaming kernel under AUTO, big M does not
-    for m in (1, 8, 32):
+    for m in (1, 8, 32, 128):
         p = capi.plan(capi.BF16BF16BF16, m, 14336, 4096, 0, 1)
         assert p.rung == capi.RUNG_SKINNY and p.grid * p.tile_n >= 14336 and p.tile_m >= m
-    assert capi.plan(capi.BF16BF16BF16, 128, 14336, 4096, 0, 1).rung == capi.RUNG_MFMA
+        # equal column groups: one or two per compute unit, 4-column granular
+        assert p.grid % 256 == 0 and p.tile_n % 4 == 0 and p.lds_bytes <= 160 * 1024
+    # the LDS-shared tile kernel is chosen only while the tiled rung cannot give every compute unit its own tile
+    assert capi.plan(capi.BF16BF16BF16, 128, 65536, 4096, 0, 1).rung == capi.RUNG_MFMA
+    assert capi.plan(capi.BF16BF16BF16, 32, 65536, 4096, 0, 1).rung == capi.RUNG_SKINNY
+    assert capi.plan(capi.BF16BF16BF16, 129, 14336, 4096, 0, 1).rung == capi.RUNG_MFMA
+    # K that is a multiple of 64 but not of 128 takes the register-streaming kernel for M <= 16
+    assert capi.plan(capi.BF16BF16BF16, 8, 4096, 192, 0, 1).tile_k == 64
+    assert capi.plan(capi.BF16BF16BF16, 8, 4096, 256, 0, 1).tile_k == 128
+    assert capi.plan(capi.BF16BF16BF16, 24, 4096, 192, 0, 1).tile_k == 64
     # a small problem shrinks the tile so that more work-groups exist
     small = capi.plan(capi.BF16BF16F32, 1024, 1024, 1024, 0, 1)
     assert small.tile_m * small.tile_n < 256 * 256

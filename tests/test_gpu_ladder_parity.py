@@ -78,8 +78,11 @@ def test_mfma_every_variant_bit_exact(G, types):
 
 @pytest.mark.parametrize("types", ALL_TYPES[1:])
 def test_skinny_rung(G, types):
+    # three kernels: M <= 16 with K % 128 == 0 (direct-to-LDS), M <= 16 otherwise (registers), 16 < M <= 128 (tile)
     for (m, n, k), (al, be) in itertools.product([(1, 16, 64), (1, 1000, 256), (8, 14336, 512), (16, 250, 128),
-                                                  (17, 33, 192), (32, 512, 4096)], [(1, 0), (0.5, 2)]):
+                                                  (13, 37, 384), (17, 33, 192), (32, 512, 4096), (33, 100, 64),
+                                                  (64, 3000, 1024), (100, 9, 128), (128, 7170, 576)],
+                                                 [(1, 0), (0.5, 2)]):
         a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=5)
         got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, al, be, SKINNY)
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, al, be)), (types, m, n, k)
@@ -92,8 +95,8 @@ def test_skinny_rung(G, types):
 
 
 def test_skinny_rung_refuses_what_it_cannot_do(G):
-    a = torch.zeros(64 * 64, dtype=torch.int16, device="cuda")
-    for kw in (dict(m=33), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32)):
+    a = torch.zeros(129 * 64, dtype=torch.int16, device="cuda")
+    for kw in (dict(m=129), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32)):
         args = dict(types=O.BF16BF16BF16, m=8, n=64, k=64, la=O.ROW, lb=O.COL)
         args.update(kw)
         with pytest.raises(G.capi.GzError) as e:

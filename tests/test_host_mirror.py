@@ -45,7 +45,7 @@ def test_constructor_plans_like_the_reference_constructors(F, capi):
 
 def test_constructor_rejects_what_the_rung_cannot_run(F, capi):
     with pytest.raises(capi.GzError) as e:
-        F.functor("skinny_gemm", "bf16", "bf16", layout_b=F.COL)(64, 128, 128)
+        F.functor("skinny_gemm", "bf16", "bf16", layout_b=F.COL)(129, 128, 128)
     assert e.value.status == capi.ERR_UNSUPPORTED
     with pytest.raises(capi.GzError):
         F.functor("naive_gemm", "bf16", "f32")(-1, 4, 4)
