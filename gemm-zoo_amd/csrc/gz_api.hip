@@ -220,7 +220,7 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
     }
     case GZ_RUNG_MFMA: {
       MfmaCfg c;
-      if (!mfma_resolve(types, m, n, k, variant, num_cus, &c)) {
+      if (!mfma_resolve(types, m, n, k, layoutA, layoutB, variant, num_cus, &c)) {
         set_error("mfma rung: unknown variant %d", variant);
         return GZ_ERR_UNSUPPORTED;
       }

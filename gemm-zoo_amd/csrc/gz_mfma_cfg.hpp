@@ -4,6 +4,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "../../include/gemm_zoo.h"
+
 namespace gz {
 
 struct MfmaCfg {
@@ -34,7 +36,8 @@ inline int mfma_lds_bytes(const MfmaCfg& c) { return 2 * (c.bm + c.bn) * MFMA_LD
 // Picks the tile configuration.  A 256x256 tile needs the fewest bytes per flop;
 // it is kept as long as the grid still covers every compute unit, otherwise the
 // tile shrinks so that more work-groups exist.
-inline bool mfma_resolve(int types, int M, int N, int /*K*/, int variant, int num_cus, MfmaCfg* out) {
+inline bool mfma_resolve(int types, int M, int N, int /*K*/, int layoutA, int layoutB, int variant, int num_cus,
+                         MfmaCfg* out) {
   if (variant < 0 || variant > kNumMfmaCfgs) return false;
   if (variant > 0) {
     *out = kMfmaCfgs[variant - 1];
@@ -48,8 +51,11 @@ inline bool mfma_resolve(int types, int M, int N, int /*K*/, int variant, int nu
   //                                           int8 8192^3  v1 543  v2 558  v5 579  v6 536  v7 582
   // The hand-scheduled kernels only exist for K-contiguous operands and whole tiles; on any other problem
   // the same tile runs the general kernel, so choosing them here is always safe.
+  // Row-major B (with row-major A) has its hand-scheduled kernel in the four-wave form only: each B fragment
+  // takes two transposing LDS reads, which fit the instruction slots of 16 MFMAs per step but not of 8.
+  const bool b_rows = layoutA == GZ_ROW_MAJOR && layoutB == GZ_ROW_MAJOR;
   if (tiles(kMfmaCfgs[0]) >= num_cus) {
-    if (types == 0) *out = kMfmaCfgs[5];                                  // int8: 4 waves, four-buffer pipeline
+    if (types == 0 || b_rows) *out = kMfmaCfgs[5];                        // 4 waves, four-buffer pipeline
     else *out = tiles(kMfmaCfgs[0]) <= 2 * num_cus ? kMfmaCfgs[6] : kMfmaCfgs[5];
   }
   else if (tiles(kMfmaCfgs[3]) >= num_cus) *out = kMfmaCfgs[3];

@@ -798,6 +798,19 @@ static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, int hand_scheduled, h
     GZ_HIP_TRY(hipGetLastError());
     return GZ_OK;
   }
+  if (!edge && akc && !bkc) {  // whole tiles, row-major A and B: direct-to-LDS copies, transposing LDS reads for B
+    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
+      if (hand_scheduled == 2) {
+        auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;
+        const size_t plds = 4u * (size_t)(BM + BN) * 64;
+        GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)plds));
+        hipLaunchKernelGGL(kern, grid, block, plds, s, g, tiles_m, tiles_n);
+        GZ_HIP_TRY(hipGetLastError());
+        return GZ_OK;
+      }
+    }
+  }
   if (edge) {
     if (akc && bkc) GZ_LAUNCH(true, true, true);
     else if (akc && !bkc) GZ_LAUNCH(true, false, true);
@@ -817,7 +830,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, int hand_scheduled, h
 template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
   using in_t = typename Traits<TYPES>::in_t;
   MfmaCfg cfg;
-  if (!mfma_resolve(TYPES, g.M, g.N, g.K, variant, 256, &cfg)) {
+  if (!mfma_resolve(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, 256, &cfg)) {
     set_error("mfma rung: unknown variant %d", variant);
     return GZ_ERR_UNSUPPORTED;
   }

@@ -20,11 +20,26 @@
 //
 // LDS rows are unpadded 64-byte rows; chunk c (16 bytes) of tile row r lives at position c ^ ((r >> 2) & 3),
 // which spreads 16 consecutive rows over the 16 four-bank groups of a 64-bank line.
+//
+// B_KC = false: B is row-major (N contiguous), the layout of the reference's own drivers.  Its half-slab then
+// sits in LDS as K rows of BN elements, filled by the same 1 KiB copies (whole K rows, so the global reads are
+// long contiguous runs), and the MFMA fragments - which want 8 (16 for int8) consecutive K values of one column
+// per lane - come out of LDS through the transposing reads ds_read_b64_tr_b16 / ds_read_b64_tr_b8: within 16
+// lanes, lane i supplies the address of 8 bytes of a [4 x 16] (b16) or [8 x 16] (b8) block, row by row, and
+// receives column i.  Two such reads make one fragment.  16-byte pieces of K row r are stored at position
+// piece ^ f(r), f(r) = (r & 3) << 2 (b16) or (r & 7) << 1 (b8), so that the rows a read touches fall into
+// different banks.
 #pragma once
 
 namespace gz {
 
 __device__ inline int pipe4_swz(int r) { return (r >> 2) & 3; }
+
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <int ES, int OFF> __device__ __forceinline__ void asm_ds_read_tr(u32x2_t& dst, uint32_t addr) {
+  if constexpr (ES == 2) asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
+  else asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
+}
 
 // copy with a lane mask: an all-zero mask turns the instruction into a no-op that still takes its place in
 // the sequence (and in the vmcnt order)
@@ -37,7 +52,7 @@ __device__ __forceinline__ void asm_copy16_masked(uint32_t voff, const void* sba
                : "memory");
 }
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_pipe4_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
@@ -52,7 +67,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr int NST = 4;              // LDS buffers
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int FM = WM / 32, FN = WN / 32;
-  constexpr int NMMA = FM * FN, NRD = FM + FN;
+  constexpr int NMMA = FM * FN, NRD = B_KC ? FM + FN : FM + 2 * FN;  // LDS reads per MFMA step
   constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (16 rows) per wave and half-slab
@@ -78,8 +93,29 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   const int lr = lane >> 2, lp = lane & 3;
   const uint32_t voff = (uint32_t)((lr * K + (lp ^ pipe4_swz(lr)) * EPV) * ES);
   const char* a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(m0 + 16 * wave * A_PW) * K * ES;
-  const char* b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 16 * wave * B_PW) * K * ES;
   const size_t group_step = (size_t)16 * K * ES;
+  // row-major B: a copy moves KRC whole K rows of the tile (BN elements each); lane -> (row, 16-byte position)
+  constexpr int KRC = 1024 / (BN * ES), LPR = 64 / KRC;  // K rows per copy, lanes per row
+  const int N = g.N;
+  uint32_t voff_b[2] = {0, 0};
+  const char* b_ubase;
+  size_t b_copy_step, b_half_step;
+  if constexpr (B_KC) {
+    b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 16 * wave * B_PW) * K * ES;
+    b_copy_step = group_step;
+    b_half_step = ROWB;
+  } else {
+    static_assert(B_KC || (KRC * BN * ES == 1024 && B_PW % 2 == 0), "whole K rows per copy");
+#pragma unroll
+    for (int par = 0; par < 2; par++) {  // copy t of the wave: rows KRC (wave B_PW + t) .., parity of t decides f(row)
+      const int kr = KRC * par + lane / LPR;   // row within a pair of copies; wave * B_PW * KRC is a multiple of 8
+      const int f = ES == 2 ? (kr & 3) << 2 : (kr & 7) << 1;
+      voff_b[par] = (uint32_t)(((size_t)(lane / LPR) * N + (size_t)(((lane % LPR) ^ f) * EPV)) * ES);
+    }
+    b_ubase = reinterpret_cast<const char*>(g.B) + ((size_t)(wave * B_PW * KRC) * N + n0) * ES;
+    b_copy_step = (size_t)KRC * N * ES;
+    b_half_step = (size_t)HK * N * ES;
+  }
   // A-row copies of half-slab hs into buffer st (one M0 for the group)
   auto copy_a_begin = [&](int st) { asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024); };
   auto copy_b_begin = [&](int st) {
@@ -91,21 +127,43 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   };
   auto copy_b = [&](auto t_c, int hs, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, OFF = (Tn - B_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(voff, b_ubase + Tn * group_step + (size_t)hs * ROWB - OFF, mask);
+    asm_copy16_masked<OFF>(B_KC ? voff : voff_b[Tn & 1], b_ubase + Tn * b_copy_step + (size_t)hs * b_half_step - OFF, mask);
   };
 
   // ---- fragment addressing: one LDS byte address per (buffer, step) ----
   const int frag_row = lane & 31, half = lane >> 5;
   const int sw = pipe4_swz(frag_row);
-  uint32_t a_addr[NST][2], b_addr[NST][2];
+  uint32_t a_addr[NST][2], b_addr[NST][B_KC ? 2 : FN];
 #pragma unroll
   for (int st = 0; st < NST; st++)
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
       const int pos = ((ks * 2 + half) ^ sw) * 16;
       a_addr[st][ks] = lds_base + st * STAGE_BYTES + (wm * WM + frag_row) * ROWB + pos;
-      b_addr[st][ks] = lds_base + st * STAGE_BYTES + A_BYTES + (wn * WN + frag_row) * ROWB + pos;
+      if constexpr (B_KC) b_addr[st][ks] = lds_base + st * STAGE_BYTES + A_BYTES + (wn * WN + frag_row) * ROWB + pos;
     }
+  // transposing reads: lane i of a 16-lane group addresses row fi of the block's K rows and the piece of 8 bytes
+  // that holds columns 16 (group & 1) + (4 or 8) (i % lanes-per-row); groups 2, 3 take the upper half of the K step.
+  // One address per (buffer, 32-column block); K step and half fragment go into the immediate offset.
+  constexpr int TR_LPR = ES == 2 ? 4 : 2;            // lanes per K row within a 16-lane group
+  constexpr int TR_PITCH = BN * ES;                   // bytes per K row
+  constexpr int TR_KS_OFF = (16 / ES * 2) * TR_PITCH; // next MFMA step: 16 (32) K rows further
+  constexpr int TR_R_OFF = (16 / TR_LPR) * TR_PITCH;  // second half fragment: 4 (8) K rows further
+  if constexpr (!B_KC) {
+    static_assert(B_KC || (TR_KS_OFF + TR_R_OFF < 65536 && TR_KS_OFF == B_BYTES / 2), "immediate offsets");
+    const int i16 = lane & 15, fi = i16 / TR_LPR;
+    const int n_sub = ((lane >> 4) & 1) * 16 + (i16 % TR_LPR) * (8 / ES);   // column within the 32-column block
+    const int krow = (lane >> 5) * (16 / TR_LPR * 2) + fi;                  // K row within the MFMA step
+    const int f = ES == 2 ? (fi & 3) << 2 : (fi & 7) << 1;
+#pragma unroll
+    for (int st = 0; st < NST; st++)
+#pragma unroll
+      for (int j = 0; j < FN; j++) {
+        const int n_local = wn * WN + j * 32 + n_sub;
+        const int piece = (n_local / EPV) ^ f;
+        b_addr[st][j] = lds_base + st * STAGE_BYTES + A_BYTES + krow * TR_PITCH + piece * 16 + (n_local % EPV) * ES;
+      }
+  }
 
   acc_v acc[FM][FN];
 #pragma unroll
@@ -120,11 +178,19 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   });
   asm volatile("s_nop 7" ::: "memory");
   u32x4_t af[2][FM], bf[2][FN];
+  u32x2_t bh[2][FN][2];  // row-major B: the two halves of a fragment as they come out of the transposing reads
 
   auto read_one = [&](auto set_c, auto r_c, int st, int ks) {
     constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value;
-    if constexpr (R < FM) asm_ds_read16<R * 32 * ROWB>(af[SET][R], a_addr[st][ks]);
-    else asm_ds_read16<(R - FM) * 32 * ROWB>(bf[SET][R - FM], b_addr[st][ks]);
+    if constexpr (R < FM) {
+      asm_ds_read16<R * 32 * ROWB>(af[SET][R], a_addr[st][ks]);
+    } else if constexpr (B_KC) {
+      asm_ds_read16<(R - FM) * 32 * ROWB>(bf[SET][R - FM], b_addr[st][ks]);
+    } else {
+      constexpr int J = (R - FM) / 2, HALF = (R - FM) % 2;
+      if (ks == 0) asm_ds_read_tr<ES, HALF * TR_R_OFF>(bh[SET][J][HALF], b_addr[st][J]);
+      else asm_ds_read_tr<ES, TR_KS_OFF + HALF * TR_R_OFF>(bh[SET][J][HALF], b_addr[st][J]);
+    }
   };
 
   // One MFMA step: NMMA MFMAs on register set SET; after MFMA q the q-th memory instruction of the step:
@@ -136,6 +202,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     constexpr int NOPS = NRD + NC;
     static_assert(NOPS <= NMMA, "one memory instruction per MFMA");
     asm volatile("s_waitcnt lgkmcnt(0)");
+    if constexpr (!B_KC) {
+#pragma unroll
+      for (int j = 0; j < FN; j++) {
+        asm volatile("" : "+v"(bh[SET][j][0]), "+v"(bh[SET][j][1]));  // after the wait
+        bf[SET][j] = u32x4_t{bh[SET][j][0][0], bh[SET][j][0][1], bh[SET][j][1][0], bh[SET][j][1][1]};
+      }
+    }
     if constexpr (IS_A) copy_a_begin(cst);
     else copy_b_begin(cst);
     static_for<NMMA>([&](auto q_c) {
@@ -206,7 +279,6 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   });
 
   // Epilogue: same register layout as the staged kernel.
-  const int N = g.N;
   const bool use_c = g.beta != 0;
 #pragma unroll
   for (int i = 0; i < FM; i++) {
