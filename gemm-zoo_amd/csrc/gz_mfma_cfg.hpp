@@ -33,33 +33,56 @@ constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
 
 inline int mfma_lds_bytes(const MfmaCfg& c) { return 2 * (c.bm + c.bn) * MFMA_LDS_PITCH; }
 
-// Picks the tile configuration.  A 256x256 tile needs the fewest bytes per flop;
-// it is kept as long as the grid still covers every compute unit, otherwise the
-// tile shrinks so that more work-groups exist.
-inline bool mfma_resolve(int types, int M, int N, int /*K*/, int layoutA, int layoutB, int variant, int num_cus,
+// Whole tiles, whole K slabs (16-byte alignment of the pointers is the caller's to check).
+inline bool mfma_whole_tiles(const MfmaCfg& c, int in_size, int M, int N, int K) {
+  const int bk = MFMA_SLAB_BYTES / in_size;
+  return K > 0 && M % c.bm == 0 && N % c.bn == 0 && K % bk == 0;
+}
+
+// Picks the tile configuration by an estimate of the launch's duration:
+//     rounds of tiles over the compute units  x  tile area  x  penalty of the tile shape  x  penalty of the kernel
+// A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does not
+// fill the device, or that leaves a nearly empty last round (N = 4097: 17 tile columns for one column of data),
+// is better served by smaller tiles.  The penalties are measured on MI355X (fp16 4095x4097x1023: 256x256 255 us,
+// 256x128 174 us, 128x128 156 us; 4096x4352x1024 row/row: 256x256 hand-scheduled 79 us, 128x128 general 103 us;
+// bf16 2048^3 row/col: 128x128 30 us, 256x128 41 us, 256x256 51 us).
+//   bf16 4096^3 (interleaved runs, us)  v1 117  v2 109  v5 108  v6 109  v7 106
+//   bf16 8192^3                         v1 904  v2 865  v6 845  v7 885
+//   int8 8192^3                         v1 543  v2 558  v5 579  v6 536  v7 582
+// Direct-to-LDS kernels exist for row-major A with whole tiles: hand-scheduled for 256x256 (column-major B: both
+// wave shapes; row-major B: four waves), compiler-scheduled for the smaller tiles; on any other problem the same
+// tile runs the general kernel, so choosing them is always safe.
+inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layoutB, int variant, int num_cus,
                          MfmaCfg* out) {
   if (variant < 0 || variant > kNumMfmaCfgs) return false;
   if (variant > 0) {
     *out = kMfmaCfgs[variant - 1];
     return true;
   }
-  auto tiles = [&](const MfmaCfg& c) {
-    return (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
-  };
-  // Measured on MI355X (interleaved runs, us): bf16 4096^3  v1 117  v2 109  v5 108  v6 109  v7 106
-  //                                           bf16 8192^3  v1 904  v2 865  v6 845  v7 885
-  //                                           int8 8192^3  v1 543  v2 558  v5 579  v6 536  v7 582
-  // The hand-scheduled kernels only exist for K-contiguous operands and whole tiles; on any other problem
-  // the same tile runs the general kernel, so choosing them here is always safe.
-  // Row-major B (with row-major A) has its hand-scheduled kernel in the four-wave form only: each B fragment
-  // takes two transposing LDS reads, which fit the instruction slots of 16 MFMAs per step but not of 8.
-  const bool b_rows = layoutA == GZ_ROW_MAJOR && layoutB == GZ_ROW_MAJOR;
-  if (tiles(kMfmaCfgs[0]) >= num_cus) {
-    if (types == 0 || b_rows) *out = kMfmaCfgs[5];                        // 4 waves, four-buffer pipeline
-    else *out = tiles(kMfmaCfgs[0]) <= 2 * num_cus ? kMfmaCfgs[6] : kMfmaCfgs[5];
+  if (num_cus <= 0) num_cus = 256;
+  const int in_size = types == 0 ? 1 : 2;
+  const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
+  // candidates: 256x256 (id 6), 256x128 (id 4), 128x128 (id 3)
+  const int cand[3] = {5, 3, 2};
+  const double shape_pen[3] = {1.0, 1.1, 1.25};
+  double best = 0;
+  int pick = 5;
+  for (int i = 0; i < 3; i++) {
+    const MfmaCfg& c = kMfmaCfgs[cand[i]];
+    const long long tiles = (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+    const long long rounds = (tiles + num_cus - 1) / num_cus;
+    const bool direct = a_rows && mfma_whole_tiles(c, in_size, M, N, K);  // every candidate has a direct-to-LDS kernel
+    const double cost = (double)rounds * c.bm * c.bn * shape_pen[i] * (direct ? 1.0 : 2.2);
+    if (i == 0 || cost < best) {
+      best = cost;
+      pick = cand[i];
+    }
   }
-  else if (tiles(kMfmaCfgs[3]) >= num_cus) *out = kMfmaCfgs[3];
-  else *out = kMfmaCfgs[2];
+  *out = kMfmaCfgs[pick];
+  if (pick == 5 && types != 0 && a_rows && b_cols) {  // 16-bit, K-contiguous B: eight waves while the grid is small
+    const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
+    if (tiles <= 2LL * num_cus) *out = kMfmaCfgs[6];
+  }
   return true;
 }
 
@@ -67,8 +90,7 @@ inline bool mfma_resolve(int types, int M, int N, int /*K*/, int layoutA, int la
 // operands; everything else runs the predicated (edge) instantiation.
 inline bool mfma_needs_edge(const MfmaCfg& c, int in_size, int /*out_size*/, int M, int N, int K, const void* A,
                             const void* B, const void* C, const void* D) {
-  const int bk = MFMA_SLAB_BYTES / in_size;
-  if (K == 0 || M % c.bm || N % c.bn || K % bk) return true;
+  if (!mfma_whole_tiles(c, in_size, M, N, K)) return true;
   const uintptr_t bits = (uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)D;
   return (bits & 15u) != 0;
 }

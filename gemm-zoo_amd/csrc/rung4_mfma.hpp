@@ -346,7 +346,27 @@ __device__ inline int dtl_swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
+// 16-byte piece c of K row r of a row-major B slab is stored at position c ^ dtl_tr_swz(r): a transposing read of
+// a 32-column block touches 4 K rows x 64 bytes (16-bit) or 8 K rows x 32 bytes (int8), and the rows of a slab are
+// a whole number of (or half a) 256-byte bank lines apart, so without this they would all hit the same banks.
+template <int ES, int PIECES_PER_ROW> __device__ inline int dtl_tr_swz(int r) {
+  static_assert(PIECES_PER_ROW >= 16 || (ES == 1 && PIECES_PER_ROW == 8), "row too short for the swizzle");
+  if constexpr (ES == 2) return (r & 3) << 2;
+  else if constexpr (PIECES_PER_ROW >= 16) return (r & 7) << 1;
+  else return ((r >> 1) & 3) << 1;
+}
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x2_t __attribute__((ext_vector_type(2)));
+// half a fragment through ds_read_b64_tr_b16 / ds_read_b64_tr_b8: lane i of 16 addresses 8 bytes of a [4 x 16]
+// ([8 x 16]) block, row by row, and receives column i
+template <int ES> __device__ inline u32x2_t lds_read_tr(const char* p) {
+  if constexpr (ES == 2)
+    return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p));
+  else
+    return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2_t*)p));
+}
+
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_dtl_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
@@ -380,12 +400,21 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // the 8-row group index q = wave*PW + t has the parity of t when PW is even; (wave*PW)&1 covers odd PW
   const in_t* a_src[2];
   const in_t* b_src[2];
+  // row-major B: the slab is BK K rows of BN elements; a copy moves KRC whole rows, LPR lanes per row
+  constexpr int TR_PITCH = BN * ES, KRC = 1024 / TR_PITCH, LPR = 64 / KRC, PPR = TR_PITCH / 16;
+  const int N = g.N;
 #pragma unroll
   for (int par = 0; par < 2; par++) {
     const int ca = lp ^ lr ^ (((wave * A_PW) & 1) ^ par);
     const int cb = lp ^ lr ^ (((wave * B_PW) & 1) ^ par);
     a_src[par] = g.A + (size_t)(m0 + 8 * wave * A_PW + lr) * K + ca * EPV;
-    b_src[par] = g.B + (size_t)(n0 + 8 * wave * B_PW + lr) * K + cb * EPV;
+    if constexpr (B_KC) {
+      b_src[par] = g.B + (size_t)(n0 + 8 * wave * B_PW + lr) * K + cb * EPV;
+    } else {
+      static_assert(B_KC || (KRC >= 4 && KRC * TR_PITCH == 1024), "the swizzle of a row must not depend on the copy index");
+      const int kr = lane / LPR;  // row within the copy; rows of a copy start at a multiple of KRC >= 4 (8 for int8)
+      b_src[par] = g.B + (size_t)(wave * B_PW * KRC + kr) * N + n0 + ((lane % LPR) ^ dtl_tr_swz<ES, PPR>(kr)) * EPV;
+    }
   }
   auto copy_slab = [&](char* stage, int k0) {
 #pragma unroll
@@ -393,9 +422,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       __builtin_amdgcn_global_load_lds((gptr_t)(a_src[t & 1] + (size_t)(8 * t) * K + k0),
                                        (lptr_t)(stage + (wave * A_PW + t) * 1024), 16, 0, 0);
 #pragma unroll
-    for (int t = 0; t < B_PW; t++)
-      __builtin_amdgcn_global_load_lds((gptr_t)(b_src[t & 1] + (size_t)(8 * t) * K + k0),
-                                       (lptr_t)(stage + A_BYTES + (wave * B_PW + t) * 1024), 16, 0, 0);
+    for (int t = 0; t < B_PW; t++) {
+      if constexpr (B_KC)
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_src[t & 1] + (size_t)(8 * t) * K + k0),
+                                         (lptr_t)(stage + A_BYTES + (wave * B_PW + t) * 1024), 16, 0, 0);
+      else
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_src[0] + (size_t)(k0 + KRC * t) * N),
+                                         (lptr_t)(stage + A_BYTES + (wave * B_PW + t) * 1024), 16, 0, 0);
+    }
   };
 
   // ---- fragment addressing ----
@@ -415,14 +449,37 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
 
+  // transposing reads of a row-major B slab: lane i of a 16-lane group addresses K row fi of the block's rows and the
+  // 8 bytes holding columns 16 (group & 1) + (4 or 8) (i % lanes-per-row); groups 2, 3 take the upper half of the step
+  constexpr int TR_LPR = ES == 2 ? 4 : 2;
+  constexpr int TR_STEP_ROWS = 32 / ES;         // K rows per MFMA step: 16 (16-bit) or 32 (int8)
+  constexpr int TR_HALF_ROWS = 16 / TR_LPR;     // K rows per transposing read: 4 or 8
+  int tr_off[FN];
+  if constexpr (!B_KC) {
+    const int i16 = lane & 15, fi = i16 / TR_LPR;
+    const int n_sub = ((lane >> 4) & 1) * 16 + (i16 % TR_LPR) * (8 / ES);
+    const int krow = (lane >> 5) * (TR_STEP_ROWS / 2) + fi;
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+      const int n_local = wn * WN + j * 32 + n_sub;
+      tr_off[j] = A_BYTES + krow * TR_PITCH + (((n_local / EPV) ^ dtl_tr_swz<ES, PPR>(fi)) * 16) + (n_local % EPV) * ES;
+    }
+  }
   u32x4_t af[2][FM], bf[2][FN];
   auto read_frags = [&](int set, const char* stage, int ks) {
 #pragma unroll
     for (int i = 0; i < FM; i++)
       af[set][i] = *reinterpret_cast<const u32x4_t*>(stage + a_base + i * 32 * ROWB + pos[ks]);
 #pragma unroll
-    for (int j = 0; j < FN; j++)
-      bf[set][j] = *reinterpret_cast<const u32x4_t*>(stage + b_base + j * 32 * ROWB + pos[ks]);
+    for (int j = 0; j < FN; j++) {
+      if constexpr (B_KC) {
+        bf[set][j] = *reinterpret_cast<const u32x4_t*>(stage + b_base + j * 32 * ROWB + pos[ks]);
+      } else {
+        const char* p = stage + tr_off[j] + ks * (TR_STEP_ROWS * TR_PITCH);
+        const u32x2_t lo = lds_read_tr<ES>(p), hi = lds_read_tr<ES>(p + TR_HALF_ROWS * TR_PITCH);
+        bf[set][j] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+      }
+    }
   };
   auto mma = [&](int set) {
 #pragma unroll
@@ -460,7 +517,6 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   }
 
   // Epilogue: same register layout as the staged kernel.
-  const int N = g.N;
   const bool use_c = g.beta != 0;
 #pragma unroll
   for (int i = 0; i < FM; i++) {
@@ -799,6 +855,15 @@ static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, int hand_scheduled, h
     return GZ_OK;
   }
   if (!edge && akc && !bkc) {  // whole tiles, row-major A and B: direct-to-LDS copies, transposing LDS reads for B
+    if constexpr (BN == 128) {
+      const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
+      auto kern = mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;
+      GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)dlds));
+      hipLaunchKernelGGL(kern, grid, block, dlds, s, g, tiles_m, tiles_n);
+      GZ_HIP_TRY(hipGetLastError());
+      return GZ_OK;
+    }
     if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;

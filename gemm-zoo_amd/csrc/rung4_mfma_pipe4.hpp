@@ -35,7 +35,6 @@ namespace gz {
 
 __device__ inline int pipe4_swz(int r) { return (r >> 2) & 3; }
 
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 template <int ES, int OFF> __device__ __forceinline__ void asm_ds_read_tr(u32x2_t& dst, uint32_t addr) {
   if constexpr (ES == 2) asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
   else asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
