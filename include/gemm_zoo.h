@@ -74,7 +74,7 @@ typedef enum gz_rung {
   GZ_RUNG_LDS_TILED = 2,       /* LDS tiles with bank-conflict-free padding        */
   GZ_RUNG_DOUBLE_BUFFERED = 3, /* global->LDS prefetch overlapped with compute     */
   GZ_RUNG_MFMA = 4,            /* wavefront-level matrix-core kernel               */
-  GZ_RUNG_SKINNY = 5,          /* weight-streaming kernel for M <= 32              */
+  GZ_RUNG_SKINNY = 5,          /* weight-streaming kernels for M <= 128            */
   GZ_NUM_RUNGS = 6
 } gz_rung;
 
