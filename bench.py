@@ -63,6 +63,8 @@ def main() -> int:
             capi.F16F16F16: torch.float16}
     OUT_T = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
              capi.F16F16F16: torch.float16}
+    OUT_DT = {capi.S8S8S32: capi.DT_INT32, capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16,
+              capi.F16F16F16: capi.DT_F16}
     IN_DT = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
              capi.F16F16F16: capi.DT_F16}
 
@@ -83,22 +85,28 @@ def main() -> int:
         return sets, d, problem_bytes
 
     def timed(types, m, n, k, la, lb, steps, warmup, rung=capi.RUNG_AUTO, variant=0, scale_b=1.0, verify=True,
-              vendor=None):
+              vendor=None, beta=0):
         sets, d, problem_bytes = make_sets(types, m, n, k, scale_b)
         p = len(sets)
+        c = None
+        if beta:  # the reference's drivers run alpha = beta = 1 (nvidia/bench/bench_bf16_mma_gemm.cu:15-16)
+            c = torch.empty(m * n, dtype=OUT_T[types], device=dev)
+            capi.fill(c, m * n, OUT_DT[types], capi.FILL_INT8_UNIFORM if types == capi.S8S8S32 else capi.FILL_NORMAL, 1.0, 4242,
+                      sptr)
+            problem_bytes += c.numel() * c.element_size()
 
         def launch(i):
             a, b = sets[i % p]
             if vendor is not None:  # the comparator library on the same operands
-                vendor(a, b, None, d, 1, 0, stream)
+                vendor(a, b, c, d, 1, beta, stream)
             else:
-                capi.gemm(types, a, b, None, d, m, n, k, la, lb, 1, 0, rung, variant, sptr)
+                capi.gemm(types, a, b, c, d, m, n, k, la, lb, 1, beta, rung, variant, sptr)
 
         if verify:  # verify-once, against an independent rung of the ladder (sequential-k LDS kernel)
             launch(0)
             ref = torch.empty_like(d)
             a, b = sets[0]
-            capi.gemm(types, a, b, None, ref, m, n, k, la, lb, 1, 0, capi.RUNG_LDS_TILED, 0, sptr)
+            capi.gemm(types, a, b, c, ref, m, n, k, la, lb, 1, beta, capi.RUNG_LDS_TILED, 0, sptr)
             if types == capi.S8S8S32:
                 ndiff = capi.compare(d, ref, m * n, capi.DT_INT32, 0.0, sptr)
             else:
@@ -178,6 +186,13 @@ def main() -> int:
         tops = 2.0 * m8 ** 3 / (r8["kernel_ms_mean"] * 1e-3) / 1e12
         extras["s8_8192"] = {"tops": round(tops, 2), "frac_of_int8_peak": round(tops / PEAK_TFLOPS["s8"], 4),
                              "kernel_ms_mean": round(r8["kernel_ms_mean"], 5)}
+        # the reference's own bench setting (alpha = beta = 1, C read as well) and its layout (row-major B)
+        rb = timed(capi.BF16BF16F32, M, N, K, capi.ROW_MAJOR, capi.COL_MAJOR, args.steps, args.warmup, beta=1)
+        extras["bf16_4096_alpha1_beta1"] = {"tflops": round(flops / (rb["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                                            "kernel_ms_mean": round(rb["kernel_ms_mean"], 5)}
+        rr = timed(capi.BF16BF16F32, M, N, K, capi.ROW_MAJOR, capi.ROW_MAJOR, args.steps, args.warmup)
+        extras["bf16_4096_row_row"] = {"tflops": round(flops / (rr["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                                       "kernel_ms_mean": round(rr["kernel_ms_mean"], 5)}
         # the vendor library beside it (the reference reports cuBLASLt): same operands, same timing, checked the same way
         try:
             functors = importlib.import_module("gemm-zoo_amd.functors")

@@ -123,3 +123,34 @@ def test_c5_skinny_bf16(G, m):
     a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=4)
     got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1, -1)
     assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1))
+
+
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16])
+@pytest.mark.parametrize("shape,tile", [((4096, 4096, 512), (256, 256)), ((2048, 4096, 1024), (256, 128)),
+                                        ((512, 384, 256), (128, 128)), ((256, 128, 128), (128, 128))])
+def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile):
+    """Row-major A and B (every driver of the reference).  The first shape gives each compute unit a whole 256x256
+    tile (hand-scheduled kernel, transposing LDS reads for B), the others take the 128-wide direct-to-LDS kernels."""
+    m, n, k = shape
+    p = G.capi.plan(types, m, n, k, O.ROW, O.ROW)
+    assert p.rung == 4 and m % p.tile_m == 0 and n % p.tile_n == 0          # whole tiles: no predicated kernel
+    assert (p.tile_m, p.tile_n) == tile
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT   # exact partial sums in any order
+    a, b, ha, hb = device_inputs(G, types, m, n, k, kind, 77)
+    hc = O.fill(m * n, O.OUT_DT[types], O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT, 1.0, 79)
+    got = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, O.ROW, 1, 1, -1)
+    rows = (0, m) if m <= 512 else (m - 24, m)
+    ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, O.ROW, 1, 1, rows=rows)
+    assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]])
+    if types != O.S8S8S32:  # N(0,1) operands against fp64 truth
+        a, b, ha, hb = device_inputs(G, types, m, n, k, O.FILL_NORMAL, 78)
+        got = G.run_gemm(types, ha, hb, None, m, n, k, O.ROW, O.ROW, 1, 0, -1)
+        truth, _ = O.gemm_f64(types, ha, hb, None, m, n, k, O.ROW, O.ROW, 1, 0, rows=(8, 24))
+        G.assert_within(types, got[8:24], truth, f"row/row {shape}")
+
+
+def test_ragged_grid_takes_the_small_tile(G):
+    # N = 4097 would need a 17th column of 256-wide tiles for one column of data
+    assert G.capi.plan(O.F16F16F16, 4095, 4097, 1023, O.ROW, O.ROW).tile_m == 128
+    assert G.capi.plan(O.BF16BF16F32, 4096, 4096, 4096, O.ROW, O.COL).tile_m == 256
+    assert G.capi.plan(O.BF16BF16F32, 2048, 2048, 2048, O.ROW, O.COL).tile_m == 128
