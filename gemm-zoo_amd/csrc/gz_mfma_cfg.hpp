@@ -33,10 +33,22 @@ constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
 
 inline int mfma_lds_bytes(const MfmaCfg& c) { return 2 * (c.bm + c.bn) * MFMA_LDS_PITCH; }
 
-// Whole tiles, whole K slabs (16-byte alignment of the pointers is the caller's to check).
+// How a problem sits on a tile configuration (16-byte alignment of the pointers is the caller's to check):
+//   WHOLE      whole tiles and whole K slabs
+//   RAGGED_MN  whole K slabs, row-major A, rows of A and B a whole number of 16-byte pieces, but M or N not a
+//              multiple of the tile: the 256x256 direct-to-LDS kernels handle it by clamping rows
+//   GENERAL    everything else: the predicated kernel
+enum { MFMA_SHAPE_WHOLE = 0, MFMA_SHAPE_RAGGED_MN = 1, MFMA_SHAPE_GENERAL = 2 };
+inline int mfma_shape_class(const MfmaCfg& c, int in_size, int M, int N, int K, int layoutA, int layoutB) {
+  const int bk = MFMA_SLAB_BYTES / in_size, epv = 16 / in_size;
+  if (K <= 0 || K % bk) return MFMA_SHAPE_GENERAL;
+  if (M % c.bm == 0 && N % c.bn == 0) return MFMA_SHAPE_WHOLE;
+  if (layoutA != GZ_ROW_MAJOR) return MFMA_SHAPE_GENERAL;
+  if (layoutB == GZ_ROW_MAJOR && N % epv) return MFMA_SHAPE_GENERAL;
+  return MFMA_SHAPE_RAGGED_MN;
+}
 inline bool mfma_whole_tiles(const MfmaCfg& c, int in_size, int M, int N, int K) {
-  const int bk = MFMA_SLAB_BYTES / in_size;
-  return K > 0 && M % c.bm == 0 && N % c.bn == 0 && K % bk == 0;
+  return mfma_shape_class(c, in_size, M, N, K, GZ_ROW_MAJOR, GZ_COL_MAJOR) == MFMA_SHAPE_WHOLE;
 }
 
 // Picks the tile configuration by an estimate of the launch's duration:
@@ -71,7 +83,9 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     const MfmaCfg& c = kMfmaCfgs[cand[i]];
     const long long tiles = (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
     const long long rounds = (tiles + num_cus - 1) / num_cus;
-    const bool direct = a_rows && mfma_whole_tiles(c, in_size, M, N, K);  // every candidate has a direct-to-LDS kernel
+    // whole tiles: every candidate has a direct-to-LDS kernel; ragged M or N: the 256x256 ones only
+    const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
+    const bool direct = a_rows && (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     const double cost = (double)rounds * c.bm * c.bn * shape_pen[i] * (direct ? 1.0 : 2.2);
     if (i == 0 || cost < best) {
       best = cost;
@@ -86,13 +100,12 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
   return true;
 }
 
-// The unpredicated kernel needs whole tiles, whole K slabs and 16-byte aligned
-// operands; everything else runs the predicated (edge) instantiation.
-inline bool mfma_needs_edge(const MfmaCfg& c, int in_size, int /*out_size*/, int M, int N, int K, const void* A,
-                            const void* B, const void* C, const void* D) {
-  if (!mfma_whole_tiles(c, in_size, M, N, K)) return true;
+// Shape class of a launch: the direct-to-LDS kernels also need 16-byte aligned operands.
+inline int mfma_launch_class(const MfmaCfg& c, int in_size, int M, int N, int K, int layoutA, int layoutB, const void* A,
+                             const void* B, const void* C, const void* D) {
   const uintptr_t bits = (uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)D;
-  return (bits & 15u) != 0;
+  if (bits & 15u) return MFMA_SHAPE_GENERAL;
+  return mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
 }
 
 }  // namespace gz

@@ -810,7 +810,7 @@ namespace gz {
 // Launcher
 // ---------------------------------------------------------------------------
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
-static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, int hand_scheduled, hipStream_t s) {
+static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_scheduled, hipStream_t s) {
   const int tiles_m = ceil_div(g.M, BM), tiles_n = ceil_div(g.N, BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(WAVES_M * WAVES_N * 64);
   const size_t lds = 2u * (size_t)(BM + BN) * PITCH;
@@ -824,6 +824,28 @@ static int launch_cfg(const GemmArgs<TYPES>& g, bool edge, int hand_scheduled, h
     hipLaunchKernelGGL(kern, grid, block, lds, s, g, tiles_m, tiles_n);                             \
   } while (0)
 
+  const bool edge = shape_class != MFMA_SHAPE_WHOLE;
+  // M or N not a multiple of the tile, everything else in order: the hand-scheduled 256x256 kernels clamp rows
+  if (shape_class == MFMA_SHAPE_RAGGED_MN && akc && hand_scheduled == 2) {
+    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+      const size_t plds = 4u * (size_t)(BM + BN) * 64;
+      if (bkc) {
+        auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>;
+        GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)plds));
+        hipLaunchKernelGGL(kern, grid, block, plds, s, g, tiles_m, tiles_n);
+        GZ_HIP_TRY(hipGetLastError());
+        return GZ_OK;
+      } else if constexpr (WAVES_N == 2) {
+        auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, true>;
+        GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)plds));
+        hipLaunchKernelGGL(kern, grid, block, plds, s, g, tiles_m, tiles_n);
+        GZ_HIP_TRY(hipGetLastError());
+        return GZ_OK;
+      }
+    }
+  }
   if (!edge && akc && bkc) {  // whole tiles, K-contiguous operands, aligned: direct-to-LDS fast path
     const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
     if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
@@ -899,8 +921,7 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipS
     set_error("mfma rung: unknown variant %d", variant);
     return GZ_ERR_UNSUPPORTED;
   }
-  const bool edge = mfma_needs_edge(cfg, (int)sizeof(in_t), (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N,
-                                    g.K, g.A, g.B, g.C, g.D);
+  const int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
   switch (cfg.id) {
     case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
     case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);

@@ -51,7 +51,7 @@ __device__ __forceinline__ void asm_copy16_masked(uint32_t voff, const void* sba
                : "memory");
 }
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true>
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true, bool RAGGED = false>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_pipe4_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
@@ -115,6 +115,36 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     b_copy_step = (size_t)KRC * N * ES;
     b_half_step = (size_t)HK * N * ES;
   }
+  // RAGGED: M and N need not be multiples of the tile (K still a whole number of slabs, rows 16-byte aligned).  Rows
+  // past the end are fetched from the last row (columns of a row-major B from its last 16-byte piece): an output
+  // depends on its own row of A and column of B only, and those past the end are not stored.  The per-copy offsets
+  // are then relative to the tile's first row instead of the copy's.
+  const int M = g.M;
+  uint32_t voff_ar[RAGGED ? A_PW : 1], voff_br[RAGGED && B_KC ? B_PW : 1];
+  const char* a_tile = reinterpret_cast<const char*>(g.A) + (size_t)m0 * K * ES;
+  const char* b_tile = reinterpret_cast<const char*>(g.B) + (size_t)n0 * K * ES;
+  if constexpr (RAGGED) {
+#pragma unroll
+    for (int t = 0; t < A_PW; t++) {
+      const int rc = min(m0 + 16 * (wave * A_PW + t) + lr, M - 1) - m0;
+      voff_ar[t] = (uint32_t)(((size_t)rc * K + (size_t)((lp ^ pipe4_swz(lr)) * EPV)) * ES);
+    }
+    if constexpr (B_KC) {
+#pragma unroll
+      for (int t = 0; t < B_PW; t++) {
+        const int rc = min(n0 + 16 * (wave * B_PW + t) + lr, N - 1) - n0;
+        voff_br[t] = (uint32_t)(((size_t)rc * K + (size_t)((lp ^ pipe4_swz(lr)) * EPV)) * ES);
+      }
+    } else {
+      const int last_piece = (N - n0) / EPV - 1;   // N is a multiple of EPV on this path, n0 < N
+#pragma unroll
+      for (int par = 0; par < 2; par++) {
+        const int kr = KRC * par + lane / LPR;
+        const int f = ES == 2 ? (kr & 3) << 2 : (kr & 7) << 1;
+        voff_b[par] = (uint32_t)(((size_t)(lane / LPR) * N + (size_t)(min((lane % LPR) ^ f, last_piece) * EPV)) * ES);
+      }
+    }
+  }
   // A-row copies of half-slab hs into buffer st (one M0 for the group)
   auto copy_a_begin = [&](int st) { asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024); };
   auto copy_b_begin = [&](int st) {
@@ -122,11 +152,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   };
   auto copy_a = [&](auto t_c, int hs, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, OFF = (Tn - A_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(voff, a_ubase + Tn * group_step + (size_t)hs * ROWB - OFF, mask);
+    if constexpr (RAGGED) asm_copy16_masked<OFF>(voff_ar[Tn], a_tile + (size_t)hs * ROWB - OFF, mask);
+    else asm_copy16_masked<OFF>(voff, a_ubase + Tn * group_step + (size_t)hs * ROWB - OFF, mask);
   };
   auto copy_b = [&](auto t_c, int hs, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, OFF = (Tn - B_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(B_KC ? voff : voff_b[Tn & 1], b_ubase + Tn * b_copy_step + (size_t)hs * b_half_step - OFF, mask);
+    if constexpr (RAGGED && B_KC) asm_copy16_masked<OFF>(voff_br[Tn], b_tile + (size_t)hs * ROWB - OFF, mask);
+    else asm_copy16_masked<OFF>(B_KC ? voff : voff_b[Tn & 1], b_ubase + Tn * b_copy_step + (size_t)hs * b_half_step - OFF, mask);
   };
 
   // ---- fragment addressing: one LDS byte address per (buffer, step) ----
@@ -288,6 +320,15 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       for (int q = 0; q < 4; q++) {
         const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
         const size_t o = (size_t)m * N + n;
+        if constexpr (RAGGED) {
+          if (m >= M || n >= N) continue;
+          if ((N & 3) != 0 || n + 3 >= N) {  // rows of D not 16-byte aligned, or the row ends inside these four
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (n + e < N) g.D[o + e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, g.C + o + e);
+            continue;
+          }
+        }
         out_t cv[4] = {0, 0, 0, 0}, dv[4];
         if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
 #pragma unroll

@@ -154,3 +154,25 @@ def test_ragged_grid_takes_the_small_tile(G):
     assert G.capi.plan(O.F16F16F16, 4095, 4097, 1023, O.ROW, O.ROW).tile_m == 128
     assert G.capi.plan(O.BF16BF16F32, 4096, 4096, 4096, O.ROW, O.COL).tile_m == 256
     assert G.capi.plan(O.BF16BF16F32, 2048, 2048, 2048, O.ROW, O.COL).tile_m == 128
+
+
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16])
+@pytest.mark.parametrize("shape,lb", [((4000, 3976, 512), O.COL), ((4000, 3976, 512), O.ROW), ((3841, 4001, 256), O.COL),
+                                      ((4090, 4080, 384), O.ROW)])
+def test_ragged_m_n_on_the_hand_scheduled_kernels(G, types, shape, lb):
+    """M and N that are not multiples of the 256x256 tile (K whole slabs, aligned rows): the direct-to-LDS kernels
+    clamp the rows they fetch and predicate the stores.  N = 4001 also makes the rows of D unaligned."""
+    m, n, k = shape
+    p = G.capi.plan(types, m, n, k, O.ROW, lb)
+    assert (p.rung, p.tile_m, p.tile_n) == (4, 256, 256)
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+    a, b, ha, hb = device_inputs(G, types, m, n, k, kind, 91)
+    hc = O.fill(m * n, O.OUT_DT[types], kind, 1.0, 93)
+    got = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, -1)
+    for rows in ((0, 8), (m - 40, m)):   # the first rows and the rows of the last, partial tile
+        ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=rows)
+        assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, shape, lb, rows)
+    # every column of the last partial tile column, a few rows spread over M
+    for r in (255, 1024, m - 1):
+        ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=(r, r + 1))
+        assert np.array_equal(got[r], ref[r])
