@@ -1,0 +1,9 @@
+// Driver of nvidia/bench/bench_rmem_64x128x128_2x4x4_f32f32f32.cu:9-24 on the functor surface of this build (fp32 x fp32 -> fp32).
+#include <tuple>
+
+#include "gemm_zoo/benchmark.hpp"
+
+int main() {
+  using kernel_functor_struct = nvidia::kernel_functors::rmem_tiled_gemm<float, float, 128, 128, 64, 16, 4, 4>;
+  benchmark::benchmark<kernel_functor_struct, float, float>({{1024, 1024, 1024}, {2048, 2048, 2048}, {4096, 4096, 4096}}, 1.0f, 1.0f);
+}

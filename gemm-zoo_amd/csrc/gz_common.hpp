@@ -50,6 +50,14 @@ template <> struct Traits<GZ_F16F16F16> {
   static constexpr bool is_int = false;
 };
 
+template <> struct Traits<GZ_F32F32F32> {
+  using in_t = float;
+  using acc_t = float;
+  using out_t = float;
+  using scalar_t = float;
+  static constexpr bool is_int = false;
+};
+
 template <int TYPES> struct GemmArgs {
   using T = Traits<TYPES>;
   const typename T::in_t* A;
@@ -83,6 +91,7 @@ __host__ __device__ inline uint16_t f32_to_f16(float f) {
 template <int TYPES> __host__ __device__ inline typename Traits<TYPES>::acc_t widen_in(typename Traits<TYPES>::in_t v) {
   if constexpr (TYPES == GZ_S8S8S32) return (int32_t)v;
   else if constexpr (TYPES == GZ_F16F16F16) return f16_to_f32(v);
+  else if constexpr (TYPES == GZ_F32F32F32) return v;
   else return bf16_to_f32(v);
 }
 
@@ -107,7 +116,7 @@ __device__ inline typename Traits<TYPES>::out_t epilogue(typename Traits<TYPES>:
     uint32_t v = (uint32_t)alpha * (uint32_t)acc;
     if (beta != 0) v += (uint32_t)beta * (uint32_t)(*c_ptr);
     return (int32_t)v;
-  } else if constexpr (TYPES == GZ_BF16BF16F32) {
+  } else if constexpr (TYPES == GZ_BF16BF16F32 || TYPES == GZ_F32F32F32) {
     float v = mul_rn(acc, alpha);
     if (beta != 0.0f) v = add_rn(v, mul_rn(beta, *c_ptr));
     return v;

@@ -72,7 +72,7 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     return true;
   }
   if (num_cus <= 0) num_cus = 256;
-  const int in_size = types == 0 ? 1 : 2;
+  const int in_size = types == GZ_S8S8S32 ? 1 : types == GZ_F32F32F32 ? 4 : 2;
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
   // candidates: 256x256 (id 6), 256x128 (id 4), 128x128 (id 3)
   const int cand[3] = {5, 3, 2};
@@ -85,7 +85,8 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     const long long rounds = (tiles + num_cus - 1) / num_cus;
     // whole tiles: every candidate has a direct-to-LDS kernel; ragged M or N: the 256x256 ones only
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
-    const bool direct = a_rows && (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
+    const bool direct = a_rows && types != GZ_F32F32F32 &&
+                        (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     const double cost = (double)rounds * c.bm * c.bn * shape_pen[i] * (direct ? 1.0 : 2.2);
     if (i == 0 || cost < best) {
       best = cost;
@@ -93,7 +94,7 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     }
   }
   *out = kMfmaCfgs[pick];
-  if (pick == 5 && types != 0 && a_rows && b_cols) {  // 16-bit, K-contiguous B: eight waves while the grid is small
+  if (pick == 5 && (types == GZ_BF16BF16F32 || types == GZ_BF16BF16BF16 || types == GZ_F16F16F16) && a_rows && b_cols) {  // 16-bit, K-contiguous B: eight waves while the grid is small
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
     if (tiles <= 2LL * num_cus) *out = kMfmaCfgs[6];
   }

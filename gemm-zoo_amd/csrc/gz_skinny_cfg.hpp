@@ -41,7 +41,7 @@ struct SkinnyCfg {
 // Decode-shaped problems only: 16-bit float inputs, activations row-major (K
 // contiguous), weights column-major (K contiguous), whole K super-steps.
 inline bool skinny_supported(int types, int M, int N, int K, int layoutA, int layoutB) {
-  if (types == GZ_S8S8S32) return false;
+  if (types != GZ_BF16BF16F32 && types != GZ_BF16BF16BF16 && types != GZ_F16F16F16) return false;
   if (layoutA != GZ_ROW_MAJOR || layoutB != GZ_COL_MAJOR) return false;
   if (M < 1 || M > SKINNY_MAX_M || N < 1 || K < SKINNY_K_STEP) return false;
   return K % SKINNY_K_STEP == 0;

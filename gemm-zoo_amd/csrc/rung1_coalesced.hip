@@ -115,5 +115,6 @@ template int launch_coalesced<GZ_S8S8S32>(const GemmArgs<GZ_S8S8S32>&, int, hipS
 template int launch_coalesced<GZ_BF16BF16F32>(const GemmArgs<GZ_BF16BF16F32>&, int, hipStream_t);
 template int launch_coalesced<GZ_BF16BF16BF16>(const GemmArgs<GZ_BF16BF16BF16>&, int, hipStream_t);
 template int launch_coalesced<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hipStream_t);
+template int launch_coalesced<GZ_F32F32F32>(const GemmArgs<GZ_F32F32F32>&, int, hipStream_t);
 
 }  // namespace gz

@@ -196,6 +196,7 @@ GZ_INST(GZ_S8S8S32)
 GZ_INST(GZ_BF16BF16F32)
 GZ_INST(GZ_BF16BF16BF16)
 GZ_INST(GZ_F16F16F16)
+GZ_INST(GZ_F32F32F32)
 #undef GZ_INST
 
 }  // namespace gz

@@ -34,6 +34,7 @@ namespace gz {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x16_t __attribute__((ext_vector_type(16)));
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -51,6 +52,15 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
   } else if constexpr (TYPES == GZ_F16F16F16) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, first),
                                                   __builtin_bit_cast(f16x8_t, second), acc, 0, 0, 0);
+  } else if constexpr (TYPES == GZ_F32F32F32) {
+    // 16 bytes per lane are 4 fp32 K values; v_mfma_f32_32x32x2_f32 takes one per lane (lanes 0-31: one k,
+    // lanes 32-63: another), so four of them consume the fragment pair.  Full fp32 products, no tf32 rounding.
+    const f32x4_t b = __builtin_bit_cast(f32x4_t, first), a = __builtin_bit_cast(f32x4_t, second);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.x, a.x, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.y, a.y, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.z, a.z, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.w, a.w, acc, 0, 0, 0);
+    return acc;
   } else {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, first),
                                                    __builtin_bit_cast(bf16x8_t, second), acc, 0, 0, 0);
@@ -143,7 +153,10 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
         const int id = u * NT + tid;
         const int mc = id % MC, ku = id / MC;
         char* dst = lds + (mc * EPV) * PITCH + ku * 4;
-        if constexpr (ES == 2) {
+        if constexpr (ES == 4) {  // one k-line per unit: element e of the vector goes to row mc * 4 + e
+#pragma unroll
+          for (int w = 0; w < 4; w++) *reinterpret_cast<uint32_t*>(dst + w * PITCH) = r[u][w];
+        } else if constexpr (ES == 2) {
           const u32x4_t lo = r[u * 2], hi = r[u * 2 + 1];
 #pragma unroll
           for (int w = 0; w < 4; w++) {
@@ -825,6 +838,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   } while (0)
 
   const bool edge = shape_class != MFMA_SHAPE_WHOLE;
+  if constexpr (TYPES != GZ_F32F32F32) {  // fp32 runs the register-staged kernel only: its MFMAs are 8x longer per byte
   // M or N not a multiple of the tile, everything else in order: the hand-scheduled 256x256 kernels clamp rows
   if (shape_class == MFMA_SHAPE_RAGGED_MN && akc && hand_scheduled == 2) {
     if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
@@ -898,6 +912,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
       }
     }
   }
+  }  // TYPES != GZ_F32F32F32
   if (edge) {
     if (akc && bkc) GZ_LAUNCH(true, true, true);
     else if (akc && !bkc) GZ_LAUNCH(true, false, true);

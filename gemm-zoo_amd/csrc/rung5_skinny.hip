@@ -538,7 +538,7 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
 }
 
 template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
-  if constexpr (TYPES == GZ_S8S8S32) {
+  if constexpr (TYPES == GZ_S8S8S32 || TYPES == GZ_F32F32F32) {
     (void)g; (void)variant; (void)s;
     set_error("skinny rung is built for the 16-bit float types only");
     return GZ_ERR_UNSUPPORTED;
@@ -585,5 +585,6 @@ template int launch_skinny<GZ_S8S8S32>(const GemmArgs<GZ_S8S8S32>&, int, hipStre
 template int launch_skinny<GZ_BF16BF16F32>(const GemmArgs<GZ_BF16BF16F32>&, int, hipStream_t);
 template int launch_skinny<GZ_BF16BF16BF16>(const GemmArgs<GZ_BF16BF16BF16>&, int, hipStream_t);
 template int launch_skinny<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hipStream_t);
+template int launch_skinny<GZ_F32F32F32>(const GemmArgs<GZ_F32F32F32>&, int, hipStream_t);
 
 }  // namespace gz

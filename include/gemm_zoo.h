@@ -21,7 +21,8 @@
  *       intel/xe_gemm_bf16_bf16_bf16_m8k16.hpp:12-47     (bf16 x bf16 -> bf16)
  *       nvidia/kernel_functors/naive_gemm.cuh:12-31, generic_gemm.cuh:14-41,
  *       smem_tiled_gemm.cuh:14-51, rmem_tiled_gemm.cuh:15-55,
- *       double_buffered_gemm.cuh:15-57, async_buffered_gemm.cuh:16-58 (ladder rungs)
+ *       double_buffered_gemm.cuh:15-57, async_buffered_gemm.cuh:16-58 (ladder rungs; the reference's
+ *       drivers for these run fp32 x fp32 -> fp32, e.g. nvidia/bench/bench_naive.cu:9-17: gz_gemm_f32f32f32)
  *   gz_plan                   <-  the functors' constructors (grid/block/LDS
  *       computation and shape checks), e.g. nvidia/kernel_functors/bf16_mma_gemm.cuh:18-49
  *   gz_fill                   <-  utils::populate_with_random nvidia/utils/fill_data.cuh:33-49,
@@ -37,6 +38,9 @@
  *                 16-bit output type: v = T(acc); v = T(v*alpha); if (beta != 0)
  *                 v = T(v + T(beta*C)) -- nvidia/kernels/generic_gemm.cuh:53-58.
  *                 alpha and beta are rounded to the output type first.
+ *   f32f32f32   : fp32 accumulate in k order with each product fused into the sum (fma), which is what the
+ *                 reference's `acc += a * b` (nvidia/kernels/naive_gemm.cuh:16-19) compiles to; epilogue as
+ *                 bf16bf16f32.  The MFMA rung uses the full-precision v_mfma_f32_32x32x2_f32, not a tf32 mode.
  */
 #ifndef GEMM_ZOO_H
 #define GEMM_ZOO_H
@@ -62,7 +66,8 @@ typedef enum gz_types {
   GZ_S8S8S32 = 0,
   GZ_BF16BF16F32 = 1,
   GZ_BF16BF16BF16 = 2,
-  GZ_F16F16F16 = 3
+  GZ_F16F16F16 = 3,
+  GZ_F32F32F32 = 4
 } gz_types;
 
 /* The ladder.  GZ_RUNG_AUTO lets the launcher pick (MFMA, or the weight-streaming
@@ -111,7 +116,11 @@ int gz_gemm_f16f16f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, u
                       int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                       float alpha, float beta, int rung, int variant, gz_stream stream);
 
-/* Type-erased form of the four above (alpha/beta as double; for s8s8s32 they must be
+int gz_gemm_f32f32f32(const float* A, const float* B, const float* C, float* D,
+                      int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                      float alpha, float beta, int rung, int variant, gz_stream stream);
+
+/* Type-erased form of the five above (alpha/beta as double; for s8s8s32 they must be
  * integral).                                                                         */
 int gz_gemm(int types, const void* A, const void* B, const void* C, void* D,
             int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,

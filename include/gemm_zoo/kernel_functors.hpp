@@ -47,6 +47,7 @@ template <> struct bundle<int8_t, int32_t> { static constexpr int value = GZ_S8S
 template <> struct bundle<bf16_t, float> { static constexpr int value = GZ_BF16BF16F32; };
 template <> struct bundle<bf16_t, bf16_t> { static constexpr int value = GZ_BF16BF16BF16; };
 template <> struct bundle<half_t, half_t> { static constexpr int value = GZ_F16F16F16; };
+template <> struct bundle<float, float> { static constexpr int value = GZ_F32F32F32; };  // the reference's ladder drivers
 
 template <typename TIn, typename TOut, layout LA, layout LB> class functor_base {
  public:
@@ -150,6 +151,18 @@ struct fp16_mma_gemm : detail::functor_base<TIn, TOut, LA, LB> {
   static_assert(std::is_same_v<TIn, half_t> && std::is_same_v<TOut, half_t>, "fp16 in and out");
   GZ_FUNCTOR_COMMON(fp16_mma_gemm, GZ_RUNG_MFMA, detail::mfma_variant_for(M, N))
 };
+
+// nvidia/kernel_functors/tf32_mma_gemm.cuh:15-60 (fp32 x fp32 -> fp32 on the tensor cores).  gfx950 has no tf32 mode;
+// the matrix-core path here is v_mfma_f32_32x32x2_f32, full fp32 products, so results are tighter than the reference's.
+template <typename TIn, typename TOut, int M = 128, int N = 128, int K = 32, layout LA = layout::row_major,
+          layout LB = layout::row_major>
+struct tf32_mma_gemm : detail::functor_base<TIn, TOut, LA, LB> {
+  static_assert(std::is_same_v<TIn, float> && std::is_same_v<TOut, float>, "fp32 in and out");
+  GZ_FUNCTOR_COMMON(tf32_mma_gemm, GZ_RUNG_MFMA, detail::mfma_variant_for(M, N))
+};
+template <typename TIn, typename TOut, int M = 128, int N = 128, int K = 32, layout LA = layout::row_major,
+          layout LB = layout::row_major>
+using f32_mma_gemm = tf32_mma_gemm<TIn, TOut, M, N, K, LA, LB>;
 
 // int8 x int8 -> int32 on the matrix cores
 template <typename TIn, typename TOut, int M = 256, int N = 256, int K = 128, layout LA = layout::row_major,

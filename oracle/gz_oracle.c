@@ -18,6 +18,10 @@
  *       val = TOut(sum)*alpha; if (beta != 0) val += beta*c   (lines 53-58)
  *       evaluated in TOut arithmetic.            -> oracle_gemm()
  *
+ *   - fp32 x fp32 -> fp32, the type of the reference's own ladder drivers (nvidia/bench/bench_naive.cu:9-17):
+ *     the same loops with each product fused into the running sum (fmaf), which is what `acc += a * b`
+ *     (nvidia/kernels/naive_gemm.cuh:16-19) compiles to under the reference's compilers' defaults.
+ *
  *   - layouts: the reference only knows row-major operands; column-major A/B
  *     is the generalisation  A(i,p) = rowmajor ? a[i*K+p] : a[p*M+i].
  *
@@ -34,6 +38,8 @@
  *                         for s8->s32 and for integer-valued float inputs;
  *                         fp64 truth within fp32 accumulation bounds; layout
  *                         probes; beta==0 never reads C.
+ *   fp32 bundle           exact rational arithmetic rounded once per step (distinguishes the fused sum from
+ *                         multiply-then-add), integer-valued inputs, fp64 truth.
  *   bf16/fp16 converters  closed-form RNE known answers, exhaustive 2^16
  *                         round trips, numpy float16 / torch bfloat16.
  *   philox4x32_10         Random123 known-answer vectors.
@@ -52,7 +58,7 @@
 
 #define ORACLE_API __attribute__((visibility("default")))
 
-enum { OR_S8S8S32 = 0, OR_BF16BF16F32 = 1, OR_BF16BF16BF16 = 2, OR_F16F16F16 = 3 };
+enum { OR_S8S8S32 = 0, OR_BF16BF16F32 = 1, OR_BF16BF16BF16 = 2, OR_F16F16F16 = 3, OR_F32F32F32 = 4 };
 enum { OR_ROW = 0, OR_COL = 1 };
 
 /* ------------------------------------------------------------------------ */
@@ -161,22 +167,25 @@ ORACLE_API void oracle_literal_f32(const float* a, const float* b, const float* 
 /* in k, exactly like the literal loop, while letting the compiler vectorise */
 /* across outputs.                                                           */
 /* ------------------------------------------------------------------------ */
-static size_t in_size(int types) { return types == OR_S8S8S32 ? 1 : 2; }
-static size_t out_size(int types) { return (types == OR_S8S8S32 || types == OR_BF16BF16F32) ? 4 : 2; }
+static size_t in_size(int types) { return types == OR_S8S8S32 ? 1 : types == OR_F32F32F32 ? 4 : 2; }
+static size_t out_size(int types) {
+  return (types == OR_S8S8S32 || types == OR_BF16BF16F32 || types == OR_F32F32F32) ? 4 : 2;
+}
 
 static float load_in_f32(int types, const void* p, size_t idx) {
+  if (types == OR_F32F32F32) return ((const float*)p)[idx];
   const uint16_t* h = (const uint16_t*)p;
   return types == OR_F16F16F16 ? oracle_f16_to_f32(h[idx]) : oracle_bf16_to_f32(h[idx]);
 }
 
 static float load_out_f32(int types, const void* p, size_t idx) {
-  if (types == OR_BF16BF16F32) return ((const float*)p)[idx];
+  if (types == OR_BF16BF16F32 || types == OR_F32F32F32) return ((const float*)p)[idx];
   if (types == OR_BF16BF16BF16) return oracle_bf16_to_f32(((const uint16_t*)p)[idx]);
   return oracle_f16_to_f32(((const uint16_t*)p)[idx]);
 }
 
 static void store_out_f32(int types, void* p, size_t idx, float v) {
-  if (types == OR_BF16BF16F32) ((float*)p)[idx] = v;
+  if (types == OR_BF16BF16F32 || types == OR_F32F32F32) ((float*)p)[idx] = v;
   else if (types == OR_BF16BF16BF16) ((uint16_t*)p)[idx] = oracle_f32_to_bf16(v);
   else ((uint16_t*)p)[idx] = oracle_f32_to_f16(v);
 }
@@ -186,7 +195,7 @@ ORACLE_API int oracle_gemm_rows(int types, const void* A, const void* B, const v
                                 int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                                 double alpha_d, double beta_d, int64_t row0, int64_t row1,
                                 int threads) {
-  if (types < 0 || types > 3 || M < 0 || N < 0 || K < 0) return 1;
+  if (types < 0 || types > OR_F32F32F32 || M < 0 || N < 0 || K < 0) return 1;
   if (row0 < 0 || row1 > M || row0 > row1) return 1;
   if (M == 0 || N == 0) return 0;
 #ifdef _OPENMP
@@ -253,8 +262,14 @@ ORACLE_API int oracle_gemm_rows(int types, const void* A, const void* B, const v
       for (int64_t p = 0; p < K; p++) {
         const float av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
         const float* brow = bf + p * N;
-        /* a*b is exact in fp32 for 16-bit inputs; one rounding per add */
-        for (int64_t j = 0; j < N; j++) acc[j] = acc[j] + av * brow[j];
+        if (types == OR_F32F32F32) {
+          /* fp32 inputs: the product is fused into the sum, which is what `acc += a * b` of the reference
+           * kernels (nvidia/kernels/naive_gemm.cuh:16-19) compiles to under nvcc's and icpx's defaults */
+          for (int64_t j = 0; j < N; j++) acc[j] = __builtin_fmaf(av, brow[j], acc[j]);
+        } else {
+          /* a*b is exact in fp32 for 16-bit inputs; one rounding per add */
+          for (int64_t j = 0; j < N; j++) acc[j] = acc[j] + av * brow[j];
+        }
       }
       for (int64_t j = 0; j < N; j++) {
         /* generic_gemm.cuh:53-58, every operation rounded to TOut */
@@ -288,7 +303,7 @@ ORACLE_API int oracle_gemm_naive_rows(int types, const void* A, const void* B, c
                                       int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                                       double alpha_d, double beta_d, int64_t row0, int64_t row1,
                                       int threads) {
-  if (types < 0 || types > 3 || M < 0 || N < 0 || K < 0) return 1;
+  if (types < 0 || types > OR_F32F32F32 || M < 0 || N < 0 || K < 0) return 1;
   if (row0 < 0 || row1 > M || row0 > row1) return 1;
   if (N == 0) return 0;
 #ifdef _OPENMP
@@ -319,7 +334,7 @@ ORACLE_API int oracle_gemm_naive_rows(int types, const void* A, const void* B, c
       for (int64_t p = 0; p < K; p++) {
         float av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
         float bv = load_in_f32(types, B, layoutB == OR_ROW ? (size_t)(p * N + j) : (size_t)(j * K + p));
-        acc = acc + av * bv;
+        acc = types == OR_F32F32F32 ? __builtin_fmaf(av, bv, acc) : acc + av * bv;
       }
       float val = round_to(types, acc);
       val = round_to(types, val * alpha);
@@ -340,7 +355,7 @@ ORACLE_API int oracle_gemm_f64(int types, const void* A, const void* B, const vo
                                double* absout, int64_t M, int64_t N, int64_t K, int layoutA,
                                int layoutB, double alpha, double beta, int64_t row0, int64_t row1,
                                int threads) {
-  if (types < 1 || types > 3) return 1;
+  if (types < 1 || types > OR_F32F32F32) return 1;
 #ifdef _OPENMP
   if (threads <= 0) threads = omp_get_max_threads();
 #else

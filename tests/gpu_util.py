@@ -10,7 +10,8 @@ import oracle_lib as O
 
 capi = importlib.import_module("gemm-zoo_amd.capi")
 
-TOL = {O.BF16BF16F32: 1e-3, O.BF16BF16BF16: 1e-2, O.F16F16F16: 1e-2}  # max relative error, BASELINE north_star
+TOL = {O.BF16BF16F32: 1e-3, O.BF16BF16BF16: 1e-2, O.F16F16F16: 1e-2,  # max relative error, BASELINE north_star
+       O.F32F32F32: 1e-4}  # fp32 inputs: only the summation order differs
 
 
 def dev():
@@ -36,7 +37,7 @@ def down(t: torch.Tensor, types: int, m: int, n: int) -> np.ndarray:
 
 
 def out_torch_dtype(types):
-    return {O.S8S8S32: torch.int32, O.BF16BF16F32: torch.float32}.get(types, torch.int16)
+    return {O.S8S8S32: torch.int32, O.BF16BF16F32: torch.float32, O.F32F32F32: torch.float32}.get(types, torch.int16)
 
 
 def run_gemm(types, a, b, c, m, n, k, la, lb, alpha, beta, rung, variant=0, misalign=0, guard=64):

@@ -11,16 +11,16 @@ ROOT = Path(__file__).resolve().parent.parent
 ORACLE_DIR = ROOT / "oracle"
 LIB = ORACLE_DIR / "liboracle.so"
 
-S8S8S32, BF16BF16F32, BF16BF16BF16, F16F16F16 = 0, 1, 2, 3
+S8S8S32, BF16BF16F32, BF16BF16BF16, F16F16F16, F32F32F32 = 0, 1, 2, 3, 4
 ROW, COL = 0, 1
-IN_DTYPE = {0: np.int8, 1: np.uint16, 2: np.uint16, 3: np.uint16}
-OUT_DTYPE = {0: np.int32, 1: np.float32, 2: np.uint16, 3: np.uint16}
+IN_DTYPE = {0: np.int8, 1: np.uint16, 2: np.uint16, 3: np.uint16, 4: np.float32}
+OUT_DTYPE = {0: np.int32, 1: np.float32, 2: np.uint16, 3: np.uint16, 4: np.float32}
 # gz_fill / oracle_fill codes
 DT_INT8, DT_BF16, DT_F16, DT_F32, DT_INT32 = 0, 1, 2, 3, 4
 NP_OF_DT = {0: np.int8, 1: np.uint16, 2: np.uint16, 3: np.float32, 4: np.int32}
 FILL_INT8_UNIFORM, FILL_NORMAL, FILL_UNIFORM_PM1, FILL_SMALL_INT = 0, 1, 2, 3
-IN_DT = {0: DT_INT8, 1: DT_BF16, 2: DT_BF16, 3: DT_F16}
-OUT_DT = {0: DT_INT32, 1: DT_F32, 2: DT_BF16, 3: DT_F16}
+IN_DT = {0: DT_INT8, 1: DT_BF16, 2: DT_BF16, 3: DT_F16, 4: DT_F32}
+OUT_DT = {0: DT_INT32, 1: DT_F32, 2: DT_BF16, 3: DT_F16, 4: DT_F32}
 
 
 def _load():

@@ -30,6 +30,8 @@ def test_version_and_names(capi):
     assert capi.lib.gz_types_name(capi.S8S8S32) == b"s8s8s32"
     assert capi.variant_count(capi.BF16BF16F32, capi.RUNG_MFMA) >= 3
     assert capi.variant_count(capi.S8S8S32, capi.RUNG_SKINNY) == 0
+    assert capi.lib.gz_types_name(capi.F32F32F32) == b"f32f32f32"
+    assert capi.variant_count(capi.F32F32F32, capi.RUNG_SKINNY) == 0 and capi.variant_count(capi.F32F32F32, capi.RUNG_MFMA) >= 3
 
 
 @pytest.mark.parametrize("kwargs,status", [
@@ -39,6 +41,7 @@ def test_version_and_names(capi):
     (dict(rung=4, variant=99), 2),
     (dict(rung=0, variant=1), 2),
     (dict(types=0, rung=5), 2),                 # no int8 streaming kernel
+    (dict(types=4, rung=5, m=8, layout_b=1), 2),  # no fp32 streaming kernel
     (dict(rung=5, m=129, layout_b=1), 2),       # M too large for the streaming kernels
     (dict(rung=5, m=8, layout_b=0), 2),         # needs column-major weights
     (dict(rung=5, m=8, layout_b=1, k=100), 2),  # K not a whole number of super-steps

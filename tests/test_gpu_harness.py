@@ -16,7 +16,7 @@ def G():
     return gpu_util
 
 
-@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16])
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32])
 def test_hipblaslt_comparator_against_oracle(G, types):
     """The comparator is only trusted after it has itself been checked: every layout pair, exact on integer data."""
     import torch
@@ -49,6 +49,10 @@ def test_harness_runs_verifies_and_reports(G, capsys):
     assert out.count("GEMM Problem: [m: ") == 2 and "GFLOPS" in out and "Time in ms" in out
     # rotating sets: a 256^3 problem needs hundreds of sets to overflow the cache; a big one needs one or two
     assert res[0].sets > 100
+    # the reference's fp32 drivers: LDS rung and the matrix-core functor that stands in for tf32_mma_gemm
+    for name in ("smem_tiled_gemm", "tf32_mma_gemm"):
+        r = H.benchmark(F.functor(name, "f32", "f32", 128, 128, 32), [(384, 256, 160)], 1.0, 1.0, num_repititions=2)[0]
+        assert r.tflops > 0
     S = F.functor("gemm_s8_s8_s32_m8k16", "s8", "s32", layout_b=F.COL)
     r = H.benchmark_sizes(S, [(512, 512, 512)], num_repititions=2)[0]
     assert r.gbps > 0

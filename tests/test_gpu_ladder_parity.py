@@ -10,7 +10,8 @@ import oracle_lib as O
 pytestmark = pytest.mark.gpu
 
 LAYOUTS = list(itertools.product((O.ROW, O.COL), repeat=2))
-ALL_TYPES = (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16)
+ALL_TYPES = (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32)
+SKINNY_TYPES = (O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16)
 VALU_RUNGS = (0, 1, 2, 3)
 MFMA = 4
 SKINNY = 5
@@ -44,7 +45,8 @@ def test_bit_exact_all_layouts_and_shapes(G, types, rung):
 @pytest.mark.parametrize("types", ALL_TYPES[1:])
 @pytest.mark.parametrize("rung", VALU_RUNGS)
 def test_valu_rungs_sum_in_k_order(G, types, rung):
-    """Rungs 0-3 add each output's products in k order, so even N(0,1) data matches the oracle bit for bit."""
+    """Rungs 0-3 add each output's products in k order (fp32 inputs: fused into the sum), so even N(0,1) data
+    matches the oracle bit for bit."""
     for (la, lb), (m, n, k) in itertools.product(LAYOUTS, [(65, 63, 129), (128, 192, 257)]):
         a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_NORMAL, seed=11)
         got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1.0, 0.5, rung)
@@ -76,7 +78,7 @@ def test_mfma_every_variant_bit_exact(G, types):
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 1, 1)), (types, variant, la, lb, m, n, k)
 
 
-@pytest.mark.parametrize("types", ALL_TYPES[1:])
+@pytest.mark.parametrize("types", SKINNY_TYPES)
 def test_skinny_rung(G, types):
     # three kernels: M <= 16 with K % 128 == 0 (direct-to-LDS), M <= 16 otherwise (registers), 16 < M <= 128 (tile)
     for (m, n, k), (al, be) in itertools.product([(1, 16, 64), (1, 1000, 256), (8, 14336, 512), (16, 250, 128),
@@ -96,7 +98,7 @@ def test_skinny_rung(G, types):
 
 def test_skinny_rung_refuses_what_it_cannot_do(G):
     a = torch.zeros(129 * 64, dtype=torch.int16, device="cuda")
-    for kw in (dict(m=129), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32)):
+    for kw in (dict(m=129), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32), dict(types=O.F32F32F32)):
         args = dict(types=O.BF16BF16BF16, m=8, n=64, k=64, la=O.ROW, lb=O.COL)
         args.update(kw)
         with pytest.raises(G.capi.GzError) as e:

@@ -19,8 +19,11 @@ def test_functor_instantiation_follows_the_reference_names(F, capi):
     assert F.functor("fp16_mma_gemm", "f16", "f16", 256, 256, 32).types == capi.F16F16F16
     assert F.functor("gemm_s8_s8_s32_m8k16", "s8", "s32").types == capi.S8S8S32
     assert F.functor("gemm_bf16_bf16_bf16_m8k16", "bf16", "bf16").types == capi.BF16BF16BF16
+    # the reference's own ladder drivers are fp32 (nvidia/bench/bench_naive.cu:9-17, bench_tf32_mma_gemm.cu:9-26)
+    assert F.functor("tf32_mma_gemm", "f32", "f32", 128, 128, 32).types == capi.F32F32F32
+    assert F.functor("naive_gemm", "f32", "f32")(128, 128, 128).plan.rung == capi.RUNG_NAIVE
     with pytest.raises(KeyError):
-        F.functor("tf32_mma_gemm", "f32", "f32")       # the fp32 ladder is outside this build
+        F.functor("fp8_mma_gemm", "f32", "f32")        # no such functor
     with pytest.raises(KeyError):
         F.functor("naive_gemm", "bf16", "s32")
 

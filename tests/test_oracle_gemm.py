@@ -204,3 +204,69 @@ def test_oracle_rows_band_and_empty():
     d = O.gemm(O.S8S8S32, a, b, c, m, n, 0, O.ROW, O.COL, 7, 2)
     assert np.array_equal(d.ravel(), 2 * c)
     assert O.gemm(O.S8S8S32, a, b, c, 0, n, k).shape == (0, n)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# fp32 x fp32 -> fp32 (the type of the reference's ladder drivers)
+# ---------------------------------------------------------------------------------------------------------
+def _round_f32(x):
+    """Exact rational -> nearest float32, ties to even (normal range only); the result as a Fraction."""
+    from fractions import Fraction
+    if x == 0:
+        return Fraction(0)
+    sign = -1 if x < 0 else 1
+    x = abs(x)
+    e = 0
+    while x >= 2:
+        x /= 2; e += 1
+    while x < 1:
+        x *= 2; e -= 1
+    assert -126 <= e <= 127
+    scaled = x * (1 << 23)                      # in [2^23, 2^24)
+    q, r = divmod(scaled.numerator, scaled.denominator)
+    twice = 2 * r
+    if twice > scaled.denominator or (twice == scaled.denominator and (q & 1)):
+        q += 1
+    return sign * Fraction(q, 1 << 23) * (Fraction(2) ** e)
+
+
+def test_oracle_f32_is_a_fused_sum_in_k_order():
+    """Each step is round(a*b + acc) with ONE rounding, in k order: exact rational arithmetic says so.  The same data
+    summed as round(round(a*b) + acc), or in another order, gives different bits (checked, so the test can tell)."""
+    from fractions import Fraction
+    rng = np.random.default_rng(7)
+    m, n, k = 3, 4, 37
+    a = rng.standard_normal(m * k).astype(np.float32)
+    b = rng.standard_normal(k * n).astype(np.float32)
+    c = rng.standard_normal(m * n).astype(np.float32)
+    got = O.gemm(O.F32F32F32, a, b, c, m, n, k, O.ROW, O.ROW, 1.0, 0.0)
+    fused = np.zeros((m, n), np.float32); unfused = np.zeros((m, n), np.float32)
+    for i in range(m):
+        for j in range(n):
+            acc = Fraction(0); acc2 = np.float32(0)
+            for p in range(k):
+                x, y = Fraction(float(a[i * k + p])), Fraction(float(b[p * n + j]))
+                acc = _round_f32(x * y + acc)
+                acc2 = np.float32(np.float32(a[i * k + p] * b[p * n + j]) + acc2)
+            fused[i, j] = np.float32(float(acc)); unfused[i, j] = acc2
+    assert np.array_equal(got, fused)
+    assert not np.array_equal(fused, unfused)
+    # the literal one-output-per-work-item loop and column-major operands give the same bits
+    assert np.array_equal(O.gemm(O.F32F32F32, a, b, c, m, n, k, O.ROW, O.ROW, 1.0, 0.0, naive=True), fused)
+    at = a.reshape(m, k).T.copy().ravel(); bt = b.reshape(k, n).T.copy().ravel()
+    assert np.array_equal(O.gemm(O.F32F32F32, at, bt, c, m, n, k, O.COL, O.COL, 1.0, 0.0), fused)
+    # epilogue: v = acc*alpha, then v + beta*c, each rounded once (as for bf16 -> f32)
+    got = O.gemm(O.F32F32F32, a, b, c, m, n, k, O.ROW, O.ROW, 1.5, -0.75)
+    want = np.float32(fused * np.float32(1.5)) + np.float32(np.float32(-0.75) * c.reshape(m, n))
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_oracle_f32_small_integers_and_fp64_truth():
+    m, n, k = 33, 65, 129
+    a, b, c = O.make_inputs(O.F32F32F32, m, n, k, kind=O.FILL_SMALL_INT, seed=5)
+    want = (a.reshape(m, k).astype(np.int64) @ b.reshape(k, n).astype(np.int64) * 2 - c.reshape(m, n).astype(np.int64))
+    assert np.array_equal(O.gemm(O.F32F32F32, a, b, c, m, n, k, O.ROW, O.ROW, 2, -1), want.astype(np.float32))
+    a, b, c = O.make_inputs(O.F32F32F32, m, n, k, seed=6)
+    truth, mag = O.gemm_f64(O.F32F32F32, a, b, c, m, n, k, O.ROW, O.COL, 1.0, 1.0)
+    got = O.gemm(O.F32F32F32, a, b, c, m, n, k, O.ROW, O.COL, 1.0, 1.0).astype(np.float64)
+    assert np.all(np.abs(got - truth) <= (k + 2) * 2.0 ** -24 * (mag + np.abs(c.reshape(m, n))))
