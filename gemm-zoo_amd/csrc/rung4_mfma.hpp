@@ -96,6 +96,26 @@ __device__ inline u32x4_t load16(const in_t* __restrict__ base, int line, int li
   }
 }
 
+// Scheduling hint for the region it closes: spread N_OTHER instructions of class MASK (0x020 global loads, 0x200 LDS
+// stores) evenly between the region's N_MFMA MFMAs instead of leaving them in one block.
+template <int MASK, int N_OTHER, int N_MFMA> __device__ inline void mix_into_mfmas() {
+  if constexpr (N_OTHER >= N_MFMA) {
+    constexpr int PER = (N_OTHER + N_MFMA - 1) / N_MFMA;
+#pragma unroll
+    for (int x = 0; x < N_MFMA; x++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(MASK, PER, 0);
+    }
+  } else {
+    constexpr int PER = N_MFMA / N_OTHER;
+#pragma unroll
+    for (int x = 0; x < N_OTHER; x++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+      __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Slab staging: global -> registers -> LDS.
 // KC == true : operand lines are K-contiguous (row-major A, column-major B).
@@ -116,6 +136,32 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
 
   u32x4_t r[VECS];
 
+  // Transposing case: which 16-byte column (mc) of which k unit (ku) a thread moves. Within a wavefront MC_LO
+  // neighbouring lanes take one contiguous run of a k line (whole 64- or 128-byte segments of global memory) and
+  // the other lane bits walk over k units, so that the dword stores of one instruction, which land EPV * PITCH
+  // bytes apart per column step, spread over the LDS banks through their k offset instead of piling onto a few.
+  // 32-bit elements are not transposed at all: a k line of the tile goes to LDS as it lies in memory (NAT_PITCH
+  // bytes per k line, lanes along the line), and the fragment reads gather one dword per k value instead.
+  static constexpr int MC_LO = 4;
+  static constexpr int NAT_PITCH = ROWS * 4 + 32;
+  __device__ static inline void unit_of(int id, int& mc, int& ku) {
+    constexpr int MC = ROWS / EPV;
+    if constexpr (ES == 4) {
+      mc = id % MC;
+      ku = id / MC;
+    } else {
+      constexpr int KU_LO = 64 / MC_LO, MC_HI = MC / MC_LO;
+      static_assert(MC % MC_LO == 0 && NT % 64 == 0, "unit mapping works on whole wavefronts");
+      const int hi = id >> 6;
+      mc = (id % MC_LO) + (hi % MC_HI) * MC_LO;
+      ku = (id & 63) / MC_LO + (hi / MC_HI) * KU_LO;
+    }
+  }
+  // LDS store instructions of one store() call
+  static constexpr int LDS_STORES = KC ? VECS : ES == 4 ? UNITS : UNITS * EPV;
+  // bytes of one staged slab of this operand
+  static constexpr int LDS_BYTES = (!KC && ES == 4) ? BK * NAT_PITCH : ROWS * PITCH;
+
   // rows_total: M or N ; row0: first tile row ; k0: first k of the slab
   __device__ inline void load(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid) {
     if constexpr (KC) {
@@ -126,11 +172,10 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
         r[it] = load16<in_t, EDGE>(base, row0 + row, rows_total, k0 + c * EPV, K);
       }
     } else {
-      constexpr int MC = ROWS / EPV;  // 16-byte columns across the tile
 #pragma unroll
       for (int u = 0; u < UNITS; u++) {
-        const int id = u * NT + tid;
-        const int mc = id % MC, ku = id / MC;
+        int mc, ku;
+        unit_of(u * NT + tid, mc, ku);
 #pragma unroll
         for (int t = 0; t < TR; t++)
           r[u * TR + t] = load16<in_t, EDGE>(base, k0 + ku * TR + t, K, row0 + mc * EPV, rows_total);
@@ -147,15 +192,13 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
         *reinterpret_cast<u32x4_t*>(lds + row * PITCH + c * 16) = r[it];
       }
     } else {
-      constexpr int MC = ROWS / EPV;
 #pragma unroll
       for (int u = 0; u < UNITS; u++) {
-        const int id = u * NT + tid;
-        const int mc = id % MC, ku = id / MC;
+        int mc, ku;
+        unit_of(u * NT + tid, mc, ku);
         char* dst = lds + (mc * EPV) * PITCH + ku * 4;
-        if constexpr (ES == 4) {  // one k-line per unit: element e of the vector goes to row mc * 4 + e
-#pragma unroll
-          for (int w = 0; w < 4; w++) *reinterpret_cast<uint32_t*>(dst + w * PITCH) = r[u][w];
+        if constexpr (ES == 4) {  // one k-line per unit, kept as it is
+          *reinterpret_cast<u32x4_t*>(lds + ku * NAT_PITCH + mc * 16) = r[u];
         } else if constexpr (ES == 2) {
           const u32x4_t lo = r[u * 2], hi = r[u * 2 + 1];
 #pragma unroll
@@ -222,7 +265,10 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int FM = WM / 32, FN = WN / 32;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA block");
-  constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
+  using StagerA = Stager<in_t, BM, NT, A_KC, EDGE>;
+  using StagerB = Stager<in_t, BN, NT, B_KC, EDGE>;
+  constexpr bool A_NAT = ES == 4 && !A_KC, B_NAT = ES == 4 && !B_KC;  // k lines kept whole in LDS
+  constexpr int A_BYTES = StagerA::LDS_BYTES, B_BYTES = StagerB::LDS_BYTES;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -234,8 +280,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  Stager<in_t, BM, NT, A_KC, EDGE> sa;
-  Stager<in_t, BN, NT, B_KC, EDGE> sb;
+  StagerA sa;
+  StagerB sb;
 
   acc_v acc[FM][FN];
 #pragma unroll
@@ -249,18 +295,39 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 
   // fragment base offsets of this lane inside a stage
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
-  const int a_off = (wm * WM + frag_row) * PITCH + frag_k;
-  const int b_off = A_BYTES + (wn * WN + frag_row) * PITCH + frag_k;
+  // (a whole-k-line operand: k value (lane / 32) * 4 + e of a step lies e lines further down, at this lane's row)
+  const int a_off = A_NAT ? (lane >> 5) * 4 * StagerA::NAT_PITCH + (wm * WM + frag_row) * 4
+                          : (wm * WM + frag_row) * PITCH + frag_k;
+  const int b_off = A_BYTES + (B_NAT ? (lane >> 5) * 4 * StagerB::NAT_PITCH + (wn * WN + frag_row) * 4
+                                     : (wn * WN + frag_row) * PITCH + frag_k);
 
   // Two fragment sets: while the MFMAs of one K step run, the ds_reads of the next are in flight.
   u32x4_t af[2][FM], bf[2][FN];
   auto read_frags = [&](int set, const char* stage, int ks) {
 #pragma unroll
-    for (int i = 0; i < FM; i++)
-      af[set][i] = *reinterpret_cast<const u32x4_t*>(stage + a_off + i * 32 * PITCH + ks * 32);
+    for (int i = 0; i < FM; i++) {
+      if constexpr (A_NAT) {
+        const char* p = stage + a_off + ks * 8 * StagerA::NAT_PITCH + i * 32 * 4;
+        af[set][i] = u32x4_t{*reinterpret_cast<const uint32_t*>(p),
+                             *reinterpret_cast<const uint32_t*>(p + StagerA::NAT_PITCH),
+                             *reinterpret_cast<const uint32_t*>(p + 2 * StagerA::NAT_PITCH),
+                             *reinterpret_cast<const uint32_t*>(p + 3 * StagerA::NAT_PITCH)};
+      } else {
+        af[set][i] = *reinterpret_cast<const u32x4_t*>(stage + a_off + i * 32 * PITCH + ks * 32);
+      }
+    }
 #pragma unroll
-    for (int j = 0; j < FN; j++)
-      bf[set][j] = *reinterpret_cast<const u32x4_t*>(stage + b_off + j * 32 * PITCH + ks * 32);
+    for (int j = 0; j < FN; j++) {
+      if constexpr (B_NAT) {
+        const char* p = stage + b_off + ks * 8 * StagerB::NAT_PITCH + j * 32 * 4;
+        bf[set][j] = u32x4_t{*reinterpret_cast<const uint32_t*>(p),
+                             *reinterpret_cast<const uint32_t*>(p + StagerB::NAT_PITCH),
+                             *reinterpret_cast<const uint32_t*>(p + 2 * StagerB::NAT_PITCH),
+                             *reinterpret_cast<const uint32_t*>(p + 3 * StagerB::NAT_PITCH)};
+      } else {
+        bf[set][j] = *reinterpret_cast<const u32x4_t*>(stage + b_off + j * 32 * PITCH + ks * 32);
+      }
+    }
   };
   auto mma = [&](int set) {
 #pragma unroll
@@ -281,32 +348,45 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   __syncthreads();
   read_frags(0, lds, 0);
 
-  // Steady state per slab (KSTEPS = 4 MFMA steps):
-  //   step 0..2 : request the fragments of the next step, then issue this step's MFMAs
-  //   after step 2: park registers (slab kt+1) -> other LDS buffer, request slab kt+2 from global memory
-  //   barrier     : every wave has written the other buffer and has finished reading this one
-  //   step 3     : request (slab kt+1, step 0) fragments from the other buffer, issue step 3 MFMAs
-  // so every LDS and global latency is covered by MFMAs, with one barrier per slab.
+  // Steady state per slab (KSTEPS = 4 MFMA steps), one barrier per slab:
+  //   step 0 : request step 1's fragments; the parked registers (slab kt+1) go to the other LDS buffer, which every
+  //            wave left before the previous barrier, one store between every few MFMAs
+  //   step 1 : request step 2's fragments; slab kt+2 is requested from global memory, again between the MFMAs
+  //   step 2 : request step 3's fragments
+  //   barrier: every wave has written the other buffer and has its last fragments of this one
+  //   step 3 : request (slab kt+1, step 0) fragments from the other buffer
+  // A wave that issues its stores and loads in one block leaves the matrix pipe idle meanwhile (it holds only a few
+  // MFMAs ahead), and all waves of the work-group would do so at the same time. The loop body is one straight line:
+  // past the end of K the predicated loads of the edge kernels fetch nothing, the others fetch the last slab again,
+  // and what is parked in LDS then is never read.
+  static_assert(KSTEPS == 4, "the slab loop is written out for four steps");
+  constexpr int MFMAS_PER_STEP = FM * FN * (ES == 4 ? 4 : 1);
   for (int kt = 0; kt < ktiles; kt++) {
     const char* cur = lds + (kt & 1) * STAGE_BYTES;
     char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS - 1; ks++) {
-      read_frags((ks + 1) & 1, cur, ks + 1);
-      mma(ks & 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (kt + 1 < ktiles) {
-      sa.store(nxt, tid);
-      sb.store(nxt + A_BYTES, tid);
-    }
-    if (kt + 2 < ktiles) {
-      sa.load(g.A, g.M, g.K, m0, (kt + 2) * BK, tid);
-      sb.load(g.B, g.N, g.K, n0, (kt + 2) * BK, tid);
-    }
+
+    read_frags(1, cur, 1);
+    sa.store(nxt, tid);
+    sb.store(nxt + A_BYTES, tid);
+    mma(0);
+    mix_into_mfmas<0x200, StagerA::LDS_STORES + StagerB::LDS_STORES, MFMAS_PER_STEP>();
+    __builtin_amdgcn_sched_barrier(0);
+
+    read_frags(0, cur, 2);
+    const int k_next = (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK;
+    sa.load(g.A, g.M, g.K, m0, k_next, tid);
+    sb.load(g.B, g.N, g.K, n0, k_next, tid);
+    mma(1);
+    mix_into_mfmas<0x020, StagerA::VECS + StagerB::VECS, MFMAS_PER_STEP>();
+    __builtin_amdgcn_sched_barrier(0);
+
+    read_frags(1, cur, 3);
+    mma(0);
+    __builtin_amdgcn_sched_barrier(0);
+
     __syncthreads();
-    if (kt + 1 < ktiles) read_frags(KSTEPS & 1, nxt, 0);
-    mma((KSTEPS - 1) & 1);
+    read_frags(0, nxt, 0);
+    mma(1);
     __builtin_amdgcn_sched_barrier(0);
   }
 
