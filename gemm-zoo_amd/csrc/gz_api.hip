@@ -26,16 +26,17 @@ int hip_fail(hipError_t e, const char* what) {
 }
 
 static const char* kRungNames[GZ_NUM_RUNGS] = {"naive", "coalesced", "lds_tiled", "double_buffered", "mfma", "skinny"};
-static const char* kTypesNames[5] = {"s8s8s32", "bf16bf16f32", "bf16bf16bf16", "f16f16f16", "f32f32f32"};
+static const char* kTypesNames[GZ_NUM_TYPES] = {"s8s8s32",   "bf16bf16f32", "bf16bf16bf16", "f16f16f16",
+                                                "f32f32f32", "e4m3e4m3f16", "e5m2e5m2f16"};
 
-static int in_size(int types) { return types == GZ_S8S8S32 ? 1 : types == GZ_F32F32F32 ? 4 : 2; }
+static int in_size(int types) { return (types == GZ_S8S8S32 || is_fp8(types)) ? 1 : types == GZ_F32F32F32 ? 4 : 2; }
 static int out_size(int types) {
   return (types == GZ_S8S8S32 || types == GZ_BF16BF16F32 || types == GZ_F32F32F32) ? 4 : 2;
 }
 
 // Shape / enum checks common to gz_plan and the GEMM entry points.
 static int check_problem(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung) {
-  if (types < 0 || types > GZ_F32F32F32) {
+  if (types < 0 || types >= GZ_NUM_TYPES) {
     set_error("unknown type bundle %d", types);
     return GZ_ERR_BAD_ARG;
   }
@@ -145,6 +146,20 @@ int gz_gemm_f32f32f32(const float* A, const float* B, const float* C, float* D, 
   return run<GZ_F32F32F32>(A, B, C, D, M, N, K, layoutA, layoutB, alpha, beta, rung, variant, stream);
 }
 
+int gz_gemm_e4m3e4m3f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, uint16_t* D, int64_t M, int64_t N,
+                        int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung, int variant,
+                        gz_stream stream) {
+  return run<GZ_E4M3E4M3F16>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<GZ_E4M3E4M3F16>(alpha),
+                             round_out<GZ_E4M3E4M3F16>(beta), rung, variant, stream);
+}
+
+int gz_gemm_e5m2e5m2f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, uint16_t* D, int64_t M, int64_t N,
+                        int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung, int variant,
+                        gz_stream stream) {
+  return run<GZ_E5M2E5M2F16>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<GZ_E5M2E5M2F16>(alpha),
+                             round_out<GZ_E5M2E5M2F16>(beta), rung, variant, stream);
+}
+
 int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K,
             int layoutA, int layoutB, double alpha, double beta, int rung, int variant, gz_stream stream) {
   switch (types) {
@@ -168,6 +183,12 @@ int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int
     case GZ_F32F32F32:
       return gz_gemm_f32f32f32((const float*)A, (const float*)B, (const float*)C, (float*)D, M, N, K, layoutA, layoutB,
                                (float)alpha, (float)beta, rung, variant, stream);
+    case GZ_E4M3E4M3F16:
+      return gz_gemm_e4m3e4m3f16((const uint8_t*)A, (const uint8_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
+                                 layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
+    case GZ_E5M2E5M2F16:
+      return gz_gemm_e5m2e5m2f16((const uint8_t*)A, (const uint8_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
+                                 layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
     default: break;
   }
   set_error("unknown type bundle %d", types);
@@ -175,11 +196,11 @@ int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int
 }
 
 int gz_variant_count(int types, int rung) {
-  if (types < 0 || types > GZ_F32F32F32) return 0;
+  if (types < 0 || types >= GZ_NUM_TYPES) return 0;
   switch (rung) {
     case GZ_RUNG_NAIVE: case GZ_RUNG_COALESCED: case GZ_RUNG_LDS_TILED: case GZ_RUNG_DOUBLE_BUFFERED: return 1;
     case GZ_RUNG_MFMA: return kNumMfmaCfgs;
-    case GZ_RUNG_SKINNY: return (types == GZ_S8S8S32 || types == GZ_F32F32F32) ? 0 : 1;
+    case GZ_RUNG_SKINNY: return (types == GZ_S8S8S32 || types == GZ_F32F32F32 || is_fp8(types)) ? 0 : 1;
     default: return 0;
   }
 }
@@ -269,7 +290,7 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
 }
 
 const char* gz_rung_name(int rung) { return (rung >= 0 && rung < GZ_NUM_RUNGS) ? kRungNames[rung] : "auto"; }
-const char* gz_types_name(int types) { return (types >= 0 && types <= GZ_F32F32F32) ? kTypesNames[types] : "?"; }
+const char* gz_types_name(int types) { return (types >= 0 && types < GZ_NUM_TYPES) ? kTypesNames[types] : "?"; }
 const char* gz_last_error(void) { return g_err; }
 int gz_version(void) { return 1; }
 

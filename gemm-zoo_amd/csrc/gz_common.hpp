@@ -58,6 +58,24 @@ template <> struct Traits<GZ_F32F32F32> {
   static constexpr bool is_int = false;
 };
 
+template <> struct Traits<GZ_E4M3E4M3F16> {
+  using in_t = uint8_t;
+  using acc_t = float;
+  using out_t = uint16_t;
+  using scalar_t = float;
+  static constexpr bool is_int = false;
+};
+template <> struct Traits<GZ_E5M2E5M2F16> {
+  using in_t = uint8_t;
+  using acc_t = float;
+  using out_t = uint16_t;
+  using scalar_t = float;
+  static constexpr bool is_int = false;
+};
+
+constexpr bool is_fp8(int types) { return types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16; }
+constexpr bool out_is_f16(int types) { return types == GZ_F16F16F16 || is_fp8(types); }
+
 template <int TYPES> struct GemmArgs {
   using T = Traits<TYPES>;
   const typename T::in_t* A;
@@ -88,8 +106,45 @@ __host__ __device__ inline uint16_t f32_to_f16(float f) {
   return __builtin_bit_cast(uint16_t, (_Float16)f);  // round-to-nearest-even
 }
 
+// ---------------------------------------------------------------------------
+// OCP 8-bit floats (device + host).  e5m2 is the upper byte of an IEEE half.  e4m3 has bias 7, no infinities,
+// one NaN code per sign (exponent and mantissa all ones) and subnormals m * 2^-9.
+// ---------------------------------------------------------------------------
+__host__ __device__ inline float e5m2_to_f32(uint8_t b) { return f16_to_f32((uint16_t)((uint16_t)b << 8)); }
+__host__ __device__ inline float e4m3_to_f32(uint8_t b) {
+  const uint32_t s = (uint32_t)(b & 0x80u) << 24, e = (b >> 3) & 15u, m = b & 7u;
+  if (e == 15u && m == 7u) return __builtin_bit_cast(float, s | 0x7fc00000u);
+  if (e == 0u) return __builtin_bit_cast(float, s | __builtin_bit_cast(uint32_t, (float)m * 0x1p-9f));
+  return __builtin_bit_cast(float, s | ((e + 120u) << 23) | (m << 20));
+}
+// fp32 -> 8-bit float with EXP exponent and MAN mantissa bits: round to nearest even, values beyond the largest
+// finite one saturate to it (also infinities), NaN gives the all-ones code.
+template <int EXP, int MAN> __host__ __device__ inline uint8_t f32_to_fp8(float f) {
+  constexpr int BIAS = (1 << (EXP - 1)) - 1;
+  // largest finite: e4m3 keeps the top exponent for numbers (mantissa 110), e5m2 gives it to inf / NaN
+  constexpr uint32_t MAX_CODE = EXP == 4 ? 0x7eu : 0x7bu;
+  const uint32_t u = __builtin_bit_cast(uint32_t, f);
+  const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint8_t)(sign | 0x7fu);
+  int e = (int)(a >> 23) - 127;
+  if (e < 1 - BIAS) e = 1 - BIAS;                   // subnormal range shares the smallest normal's spacing
+  if (e > BIAS + 1) return (uint8_t)(sign | MAX_CODE);
+  // spacing of the target format around |f| is 2^(e - MAN); scaling by a power of two is exact
+  const float inv_ulp = __builtin_bit_cast(float, (uint32_t)(127 - (e - MAN)) << 23);
+  const uint32_t q = (uint32_t)__builtin_rintf(__builtin_bit_cast(float, a) * inv_ulp);  // 0 .. 2^(MAN+1)
+  // q counts spacings from zero of this binade's grid: code = ((e + BIAS - 1) << MAN) + q also carries a
+  // rounding up into the next binade and the subnormal / normal boundary
+  const uint32_t code = ((uint32_t)(e + BIAS - 1) << MAN) + q;
+  return (uint8_t)(sign | (code > MAX_CODE ? MAX_CODE : code));
+}
+__host__ __device__ inline uint8_t f32_to_e4m3(float f) { return f32_to_fp8<4, 3>(f); }
+__host__ __device__ inline uint8_t f32_to_e5m2(float f) { return f32_to_fp8<5, 2>(f); }
+
 template <int TYPES> __host__ __device__ inline typename Traits<TYPES>::acc_t widen_in(typename Traits<TYPES>::in_t v) {
   if constexpr (TYPES == GZ_S8S8S32) return (int32_t)v;
+  else if constexpr (TYPES == GZ_E4M3E4M3F16) return e4m3_to_f32(v);
+  else if constexpr (TYPES == GZ_E5M2E5M2F16) return e5m2_to_f32(v);
   else if constexpr (TYPES == GZ_F16F16F16) return f16_to_f32(v);
   else if constexpr (TYPES == GZ_F32F32F32) return v;
   else return bf16_to_f32(v);
@@ -97,7 +152,7 @@ template <int TYPES> __host__ __device__ inline typename Traits<TYPES>::acc_t wi
 
 template <int TYPES> __host__ __device__ inline float round_out(float v) {
   if constexpr (TYPES == GZ_BF16BF16BF16) return bf16_to_f32(f32_to_bf16(v));
-  else if constexpr (TYPES == GZ_F16F16F16) return f16_to_f32(f32_to_f16(v));
+  else if constexpr (out_is_f16(TYPES)) return f16_to_f32(f32_to_f16(v));
   else return v;
 }
 
@@ -162,7 +217,7 @@ int hip_fail(hipError_t e, const char* what);
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// Launchers, one per rung, explicitly instantiated for the four type bundles in
+// Launchers, one per rung, explicitly instantiated for every type bundle in
 // the rung's own translation unit.  Each returns a gz_status.
 template <int TYPES> int launch_naive(const GemmArgs<TYPES>& g, int variant, hipStream_t s);
 template <int TYPES> int launch_coalesced(const GemmArgs<TYPES>& g, int variant, hipStream_t s);

@@ -109,6 +109,8 @@ __global__ void __launch_bounds__(256) fill_kernel(void* dst, int64_t count, int
       case 1: static_cast<uint16_t*>(dst)[i] = f32_to_bf16(v); break;
       case 2: static_cast<uint16_t*>(dst)[i] = f32_to_f16(v); break;
       case 3: static_cast<float*>(dst)[i] = v; break;
+      case 5: static_cast<uint8_t*>(dst)[i] = f32_to_e4m3(v); break;
+      case 6: static_cast<uint8_t*>(dst)[i] = f32_to_e5m2(v); break;
       default: static_cast<int32_t*>(dst)[i] = (int32_t)v; break;
     }
   }
@@ -151,7 +153,7 @@ using namespace gz;
 extern "C" {
 
 int gz_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t seed, gz_stream stream) {
-  if (count < 0 || dtype < 0 || dtype > 4 || kind < 0 || kind > 3) {
+  if (count < 0 || dtype < 0 || dtype > 6 || kind < 0 || kind > 3) {
     set_error("gz_fill: bad argument (count=%lld dtype=%d kind=%d)", (long long)count, dtype, kind);
     return GZ_ERR_BAD_ARG;
   }

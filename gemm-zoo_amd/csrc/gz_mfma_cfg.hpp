@@ -72,7 +72,7 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     return true;
   }
   if (num_cus <= 0) num_cus = 256;
-  const int in_size = types == GZ_S8S8S32 ? 1 : types == GZ_F32F32F32 ? 4 : 2;
+  const int in_size = (types == GZ_S8S8S32 || types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) ? 1 : types == GZ_F32F32F32 ? 4 : 2;
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
   // candidates: 256x256 (id 6), 256x128 (id 4), 128x128 (id 3)
   const int cand[3] = {5, 3, 2};

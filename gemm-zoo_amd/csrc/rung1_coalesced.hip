@@ -116,5 +116,7 @@ template int launch_coalesced<GZ_BF16BF16F32>(const GemmArgs<GZ_BF16BF16F32>&, i
 template int launch_coalesced<GZ_BF16BF16BF16>(const GemmArgs<GZ_BF16BF16BF16>&, int, hipStream_t);
 template int launch_coalesced<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hipStream_t);
 template int launch_coalesced<GZ_F32F32F32>(const GemmArgs<GZ_F32F32F32>&, int, hipStream_t);
+template int launch_coalesced<GZ_E4M3E4M3F16>(const GemmArgs<GZ_E4M3E4M3F16>&, int, hipStream_t);
+template int launch_coalesced<GZ_E5M2E5M2F16>(const GemmArgs<GZ_E5M2E5M2F16>&, int, hipStream_t);
 
 }  // namespace gz

@@ -197,6 +197,8 @@ GZ_INST(GZ_BF16BF16F32)
 GZ_INST(GZ_BF16BF16BF16)
 GZ_INST(GZ_F16F16F16)
 GZ_INST(GZ_F32F32F32)
+GZ_INST(GZ_E4M3E4M3F16)
+GZ_INST(GZ_E5M2E5M2F16)
 #undef GZ_INST
 
 }  // namespace gz

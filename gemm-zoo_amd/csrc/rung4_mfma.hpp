@@ -52,6 +52,20 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
   } else if constexpr (TYPES == GZ_F16F16F16) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, first),
                                                   __builtin_bit_cast(f16x8_t, second), acc, 0, 0, 0);
+  } else if constexpr (is_fp8(TYPES)) {
+    // 16 bytes per lane are 16 K values; v_mfma_f32_32x32x16_{fp8_fp8,bf8_bf8} takes 8 per lane, so the two halves
+    // of the fragment pair feed one instruction each (which k a lane's bytes stand for is the same on both
+    // operands, and that is all a dot product needs).
+    typedef long i64x2_t __attribute__((ext_vector_type(2)));
+    const i64x2_t b = __builtin_bit_cast(i64x2_t, first), a = __builtin_bit_cast(i64x2_t, second);
+    if constexpr (TYPES == GZ_E4M3E4M3F16) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(b.x, a.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(b.y, a.y, acc, 0, 0, 0);
+    } else {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(b.x, a.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(b.y, a.y, acc, 0, 0, 0);
+    }
+    return acc;
   } else if constexpr (TYPES == GZ_F32F32F32) {
     // 16 bytes per lane are 4 fp32 K values; v_mfma_f32_32x32x2_f32 takes one per lane (lanes 0-31: one k,
     // lanes 32-63: another), so four of them consume the fragment pair.  Full fp32 products, no tf32 rounding.
@@ -66,6 +80,9 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
                                                    __builtin_bit_cast(bf16x8_t, second), acc, 0, 0, 0);
   }
 }
+
+// MFMA instructions behind one mfma32 call
+template <int TYPES> constexpr int mfmas_per_fragment() { return TYPES == GZ_F32F32F32 ? 4 : is_fp8(TYPES) ? 2 : 1; }
 
 constexpr int SLAB_BYTES = 128;           // K bytes per tile row per slab
 constexpr int PITCH = SLAB_BYTES + 16;    // LDS row pitch
@@ -360,7 +377,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // past the end of K the predicated loads of the edge kernels fetch nothing, the others fetch the last slab again,
   // and what is parked in LDS then is never read.
   static_assert(KSTEPS == 4, "the slab loop is written out for four steps");
-  constexpr int MFMAS_PER_STEP = FM * FN * (ES == 4 ? 4 : 1);
+  constexpr int MFMAS_PER_STEP = FM * FN * mfmas_per_fragment<TYPES>();
   for (int kt = 0; kt < ktiles; kt++) {
     const char* cur = lds + (kt & 1) * STAGE_BYTES;
     char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
@@ -918,10 +935,13 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   } while (0)
 
   const bool edge = shape_class != MFMA_SHAPE_WHOLE;
+  // the fixed instruction sequences are written for one MFMA per fragment pair; the 8-bit float types run the
+  // compiler-scheduled direct-to-LDS kernel on whole tiles
+  constexpr bool HAND_SCHEDULED = !is_fp8(TYPES);
   if constexpr (TYPES != GZ_F32F32F32) {  // fp32 runs the register-staged kernel only: its MFMAs are 8x longer per byte
   // M or N not a multiple of the tile, everything else in order: the hand-scheduled 256x256 kernels clamp rows
   if (shape_class == MFMA_SHAPE_RAGGED_MN && akc && hand_scheduled == 2) {
-    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
       const size_t plds = 4u * (size_t)(BM + BN) * 64;
       if (bkc) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>;
@@ -942,7 +962,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   }
   if (!edge && akc && bkc) {  // whole tiles, K-contiguous operands, aligned: direct-to-LDS fast path
     const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
-    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
         const size_t plds = 4u * (size_t)(BM + BN) * 64;
@@ -953,7 +973,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
         return GZ_OK;
       }
     }
-    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
+    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
       if (hand_scheduled == 1) {
         auto kern = mfma_asm_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
         GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -980,7 +1000,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
       GZ_HIP_TRY(hipGetLastError());
       return GZ_OK;
     }
-    if constexpr (BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
+    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;
         const size_t plds = 4u * (size_t)(BM + BN) * 64;

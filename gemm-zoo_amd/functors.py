@@ -18,7 +18,8 @@ ROW, COL = capi.ROW_MAJOR, capi.COL_MAJOR
 
 # (TIn, TOut) -> type bundle, spelled as in the reference's drivers
 BUNDLES = {("s8", "s32"): capi.S8S8S32, ("bf16", "f32"): capi.BF16BF16F32, ("bf16", "bf16"): capi.BF16BF16BF16,
-           ("f16", "f16"): capi.F16F16F16, ("f32", "f32"): capi.F32F32F32}
+           ("f16", "f16"): capi.F16F16F16, ("f32", "f32"): capi.F32F32F32,
+           ("e4m3", "f16"): capi.E4M3E4M3F16, ("e5m2", "f16"): capi.E5M2E5M2F16}
 
 # functor name -> (rung, tile ints -> variant)
 _RUNGS = {
@@ -33,6 +34,7 @@ _RUNGS = {
     "tf32_mma_gemm": capi.RUNG_MFMA,              # nvidia/kernel_functors/tf32_mma_gemm.cuh:15 (full fp32 MFMA here)
     "f32_mma_gemm": capi.RUNG_MFMA,
     "fp16_mma_gemm": capi.RUNG_MFMA,
+    "fp8_mma_gemm": capi.RUNG_MFMA,               # no counterpart: the reference runs fp8 through cuBLASLt only
     "s8_mma_gemm": capi.RUNG_MFMA,
     "gemm_s8_s8_s32_m8k16": capi.RUNG_AUTO,       # intel/xe_gemm_s8_s8_s32_m8k16.hpp:12
     "gemm_bf16_bf16_f32_m8k16": capi.RUNG_AUTO,   # intel/xe_gemm_bf16_bf16_f32_m8k16.hpp:12

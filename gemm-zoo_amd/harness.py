@@ -30,16 +30,20 @@ def _torch_types(types):
     import torch
 
     tin = {capi.S8S8S32: torch.int8, capi.BF16BF16F32: torch.bfloat16, capi.BF16BF16BF16: torch.bfloat16,
-           capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32}[types]
+           capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32,
+           capi.E4M3E4M3F16: torch.float8_e4m3fn, capi.E5M2E5M2F16: torch.float8_e5m2}[types]
     tout = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
-            capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32}[types]
+            capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32,
+            capi.E4M3E4M3F16: torch.float16, capi.E5M2E5M2F16: torch.float16}[types]
     return tin, tout
 
 
 _IN_DT = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
-          capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32}
+          capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32,
+          capi.E4M3E4M3F16: capi.DT_E4M3, capi.E5M2E5M2F16: capi.DT_E5M2}
 _OUT_DT = {capi.S8S8S32: capi.DT_INT32, capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16,
-           capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32}
+           capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32,
+           capi.E4M3E4M3F16: capi.DT_F16, capi.E5M2E5M2F16: capi.DT_F16}
 
 
 def benchmark_impl(kernel_cls, m, n, k, alpha, beta, stream=None, num_repititions=50, verify=True, quiet=False):

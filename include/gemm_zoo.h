@@ -38,6 +38,10 @@
  *                 16-bit output type: v = T(acc); v = T(v*alpha); if (beta != 0)
  *                 v = T(v + T(beta*C)) -- nvidia/kernels/generic_gemm.cuh:53-58.
  *                 alpha and beta are rounded to the output type first.
+ *   e4m3e4m3f16, e5m2e5m2f16 : inputs are OCP 8-bit floats (e4m3: bias 7, no infinities, 0x7f/0xff NaN, largest
+ *                 448; e5m2: the upper byte of an IEEE half); every product is exact in fp32; fp32 accumulate;
+ *                 epilogue in fp16 as for f16f16f16 (the reference's checker computes these types in float,
+ *                 nvidia/kernels/generic_gemm.cuh:10-13,53-58).
  *   f32f32f32   : fp32 accumulate in k order with each product fused into the sum (fma), which is what the
  *                 reference's `acc += a * b` (nvidia/kernels/naive_gemm.cuh:16-19) compiles to; epilogue as
  *                 bf16bf16f32.  The MFMA rung uses the full-precision v_mfma_f32_32x32x2_f32, not a tf32 mode.
@@ -67,7 +71,10 @@ typedef enum gz_types {
   GZ_BF16BF16F32 = 1,
   GZ_BF16BF16BF16 = 2,
   GZ_F16F16F16 = 3,
-  GZ_F32F32F32 = 4
+  GZ_F32F32F32 = 4,
+  GZ_E4M3E4M3F16 = 5, /* OCP fp8 e4m3 (finite-only, __nv_fp8_e4m3's format) x e4m3 -> fp16 */
+  GZ_E5M2E5M2F16 = 6, /* OCP fp8 e5m2 (__nv_fp8_e5m2's format) x e5m2 -> fp16            */
+  GZ_NUM_TYPES = 7
 } gz_types;
 
 /* The ladder.  GZ_RUNG_AUTO lets the launcher pick (MFMA, or the weight-streaming
@@ -120,7 +127,19 @@ int gz_gemm_f32f32f32(const float* A, const float* B, const float* C, float* D,
                       int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                       float alpha, float beta, int rung, int variant, gz_stream stream);
 
-/* Type-erased form of the five above (alpha/beta as double; for s8s8s32 they must be
+/* fp8 inputs (one byte per element, raw bit patterns), fp16 output: the bundles of the reference's
+ * cublasLt_gemm<__nv_fp8_e4m3, __half> / <__nv_fp8_e5m2, __half> (nvidia/kernel_functors/cublaslt_gemm.cuh,
+ * nvidia/bench/bench_cublaslt_e4m3.cu:6-21, bench_cublaslt_e5m2.cu:6-21), which the reference only runs through
+ * cuBLASLt; here they have kernels of their own on every rung.                                              */
+int gz_gemm_e4m3e4m3f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, uint16_t* D,
+                        int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                        float alpha, float beta, int rung, int variant, gz_stream stream);
+
+int gz_gemm_e5m2e5m2f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, uint16_t* D,
+                        int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                        float alpha, float beta, int rung, int variant, gz_stream stream);
+
+/* Type-erased form of the typed entry points above (alpha/beta as double; for s8s8s32 they must be
  * integral).                                                                         */
 int gz_gemm(int types, const void* A, const void* B, const void* C, void* D,
             int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
@@ -138,7 +157,8 @@ const char* gz_types_name(int types);
 
 /* Seeded device fill: element i of `dst` is a pure function of (seed, i) through
  * Philox4x32-10 with counter = i and key = seed.
- *   dtype: 0 int8, 1 bf16, 2 fp16, 3 fp32, 4 int32
+ *   dtype: 0 int8, 1 bf16, 2 fp16, 3 fp32, 4 int32, 5 fp8 e4m3, 6 fp8 e5m2 (round to nearest even,
+ *          saturating to the largest finite value)
  *   kind : 0 integers uniform in [-128,127]   1 N(0,1)*scale   2 U(-1,1)*scale
  *          3 small integers in {-1,0,1} (exactly representable partial sums)      */
 int gz_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t seed,
@@ -148,7 +168,7 @@ int gz_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t
  * of the stored values; otherwise |out - ref| > abs_threshold counts as different.
  * Synchronises `stream`.  *num_different (host memory, may be NULL) receives the count.
  * Returns GZ_ERR_MISMATCH if any element differs.
- *   dtype as in gz_fill.                                                            */
+ *   dtype as in gz_fill (0..4; 8-bit floats are inputs only).                        */
 int gz_compare(const void* out, const void* ref, int64_t count, int dtype,
                float abs_threshold, int64_t* num_different, gz_stream stream);
 

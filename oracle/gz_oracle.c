@@ -22,6 +22,13 @@
  *     the same loops with each product fused into the running sum (fmaf), which is what `acc += a * b`
  *     (nvidia/kernels/naive_gemm.cuh:16-19) compiles to under the reference's compilers' defaults.
  *
+ *   - fp8 x fp8 -> fp16 (nvidia/bench/bench_cublaslt_e4m3.cu:6-21, bench_cublaslt_e5m2.cu:6-21: __nv_fp8_e4m3 /
+ *     __nv_fp8_e5m2 inputs, __half output): the reference has no kernel of its own for these, only cuBLASLt and the
+ *     generic checker, which "does all the compute in float" (nvidia/kernels/generic_gemm.cuh:10-13): the same
+ *     oracle_gemm() loop on decoded inputs with the fp16 epilogue.  The two formats are the OCP 8-bit floats
+ *     (OCP 8-bit Floating Point Specification v1.0): e4m3 = 1-4-3 bits, bias 7, no infinities, S.1111.111 NaN,
+ *     largest finite 448; e5m2 = 1-5-2 bits, bias 15, IEEE-style infinities and NaNs.   -> oracle_fp8_*()
+ *
  *   - layouts: the reference only knows row-major operands; column-major A/B
  *     is the generalisation  A(i,p) = rowmajor ? a[i*K+p] : a[p*M+i].
  *
@@ -40,6 +47,11 @@
  *                         probes; beta==0 never reads C.
  *   fp32 bundle           exact rational arithmetic rounded once per step (distinguishes the fused sum from
  *                         multiply-then-add), integer-valued inputs, fp64 truth.
+ *   fp8 decode / encode   every one of the 256 codes of both formats against torch.float8_e4m3fn / float8_e5m2
+ *                         (an independent implementation), the specification's table of extreme values,
+ *                         encode(decode(code)) == code, ties-to-even and saturation known answers; the GEMM
+ *                         on fp8 inputs against exact integer arithmetic (every product and partial sum of
+ *                         small codes is exact) and fp64 truth.
  *   bf16/fp16 converters  closed-form RNE known answers, exhaustive 2^16
  *                         round trips, numpy float16 / torch bfloat16.
  *   philox4x32_10         Random123 known-answer vectors.
@@ -58,7 +70,8 @@
 
 #define ORACLE_API __attribute__((visibility("default")))
 
-enum { OR_S8S8S32 = 0, OR_BF16BF16F32 = 1, OR_BF16BF16BF16 = 2, OR_F16F16F16 = 3, OR_F32F32F32 = 4 };
+enum { OR_S8S8S32 = 0, OR_BF16BF16F32 = 1, OR_BF16BF16BF16 = 2, OR_F16F16F16 = 3, OR_F32F32F32 = 4,
+       OR_E4M3E4M3F16 = 5, OR_E5M2E5M2F16 = 6, OR_NUM_TYPES = 7 };
 enum { OR_ROW = 0, OR_COL = 1 };
 
 /* ------------------------------------------------------------------------ */
@@ -120,9 +133,47 @@ ORACLE_API uint16_t oracle_f32_to_f16(float f) {
   return (uint16_t)(sign | (base + q)); /* carry into exponent is intended */
 }
 
+/* ------------------------------------------------------------------------ */
+/* OCP 8-bit floats, from the format definition:                             */
+/*   normal     (-1)^s * 2^(E - bias) * (1 + m / 2^MAN)      1 <= E          */
+/*   subnormal  (-1)^s * 2^(1 - bias) * (m / 2^MAN)          E == 0          */
+/* e4m3 (bias 7): E == 15 is an ordinary exponent, except S.1111.111 = NaN.  */
+/* e5m2 (bias 15): E == 31 is infinity (m == 0) or NaN.                      */
+/* ------------------------------------------------------------------------ */
+ORACLE_API float oracle_fp8_to_f32(int e5m2, uint8_t code) {
+  const int man_bits = e5m2 ? 2 : 3, bias = e5m2 ? 15 : 7;
+  const int sign = code >> 7, E = (code & 0x7f) >> man_bits, m = code & ((1 << man_bits) - 1);
+  float mag;
+  if (e5m2 && E == 31) mag = m ? NAN : INFINITY;
+  else if (!e5m2 && E == 15 && m == 7) mag = NAN;
+  else if (E == 0) mag = ldexpf((float)m, 1 - bias - man_bits);
+  else mag = ldexpf((float)((1 << man_bits) + m), E - bias - man_bits);
+  return sign ? -mag : mag;
+}
+
+/* Nearest finite code, ties to the code with an even mantissa, beyond the largest finite value: that value
+ * (the saturating conversion; what the device fill uses).  Found by search over the 2^7 magnitudes, which is
+ * slow and obviously right.                                                                                */
+ORACLE_API uint8_t oracle_f32_to_fp8(int e5m2, float f) {
+  const uint8_t sign = signbit(f) ? 0x80 : 0;
+  if (isnan(f)) return (uint8_t)(sign | 0x7f);
+  const uint8_t max_code = e5m2 ? 0x7b : 0x7e;
+  const double a = fabs((double)f);
+  if (isinf(f) || a >= (double)oracle_fp8_to_f32(e5m2, max_code)) return (uint8_t)(sign | max_code);
+  uint8_t best = 0;
+  double best_err = a; /* distance to code 0 */
+  for (int c = 1; c <= max_code; c++) {
+    const double err = fabs(a - (double)oracle_fp8_to_f32(e5m2, (uint8_t)c));
+    if (err < best_err || (err == best_err && (c & 1) == 0)) { best = (uint8_t)c; best_err = err; }
+  }
+  return (uint8_t)(sign | best);
+}
+
+static inline int is_fp8(int types) { return types == OR_E4M3E4M3F16 || types == OR_E5M2E5M2F16; }
+
 static inline float round_to(int types, float v) {
   if (types == OR_BF16BF16BF16) return oracle_bf16_to_f32(oracle_f32_to_bf16(v));
-  if (types == OR_F16F16F16) return oracle_f16_to_f32(oracle_f32_to_f16(v));
+  if (types == OR_F16F16F16 || is_fp8(types)) return oracle_f16_to_f32(oracle_f32_to_f16(v));
   return v;
 }
 
@@ -167,13 +218,17 @@ ORACLE_API void oracle_literal_f32(const float* a, const float* b, const float* 
 /* in k, exactly like the literal loop, while letting the compiler vectorise */
 /* across outputs.                                                           */
 /* ------------------------------------------------------------------------ */
-static size_t in_size(int types) { return types == OR_S8S8S32 ? 1 : types == OR_F32F32F32 ? 4 : 2; }
+static size_t in_size(int types) {
+  return (types == OR_S8S8S32 || types == OR_E4M3E4M3F16 || types == OR_E5M2E5M2F16) ? 1 : types == OR_F32F32F32 ? 4 : 2;
+}
 static size_t out_size(int types) {
   return (types == OR_S8S8S32 || types == OR_BF16BF16F32 || types == OR_F32F32F32) ? 4 : 2;
 }
 
 static float load_in_f32(int types, const void* p, size_t idx) {
   if (types == OR_F32F32F32) return ((const float*)p)[idx];
+  if (types == OR_E4M3E4M3F16) return oracle_fp8_to_f32(0, ((const uint8_t*)p)[idx]);
+  if (types == OR_E5M2E5M2F16) return oracle_fp8_to_f32(1, ((const uint8_t*)p)[idx]);
   const uint16_t* h = (const uint16_t*)p;
   return types == OR_F16F16F16 ? oracle_f16_to_f32(h[idx]) : oracle_bf16_to_f32(h[idx]);
 }
@@ -195,7 +250,7 @@ ORACLE_API int oracle_gemm_rows(int types, const void* A, const void* B, const v
                                 int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                                 double alpha_d, double beta_d, int64_t row0, int64_t row1,
                                 int threads) {
-  if (types < 0 || types > OR_F32F32F32 || M < 0 || N < 0 || K < 0) return 1;
+  if (types < 0 || types >= OR_NUM_TYPES || M < 0 || N < 0 || K < 0) return 1;
   if (row0 < 0 || row1 > M || row0 > row1) return 1;
   if (M == 0 || N == 0) return 0;
 #ifdef _OPENMP
@@ -303,7 +358,7 @@ ORACLE_API int oracle_gemm_naive_rows(int types, const void* A, const void* B, c
                                       int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                                       double alpha_d, double beta_d, int64_t row0, int64_t row1,
                                       int threads) {
-  if (types < 0 || types > OR_F32F32F32 || M < 0 || N < 0 || K < 0) return 1;
+  if (types < 0 || types >= OR_NUM_TYPES || M < 0 || N < 0 || K < 0) return 1;
   if (row0 < 0 || row1 > M || row0 > row1) return 1;
   if (N == 0) return 0;
 #ifdef _OPENMP
@@ -355,7 +410,7 @@ ORACLE_API int oracle_gemm_f64(int types, const void* A, const void* B, const vo
                                double* absout, int64_t M, int64_t N, int64_t K, int layoutA,
                                int layoutB, double alpha, double beta, int64_t row0, int64_t row1,
                                int threads) {
-  if (types < 1 || types > OR_F32F32F32) return 1;
+  if (types < 1 || types >= OR_NUM_TYPES) return 1;
 #ifdef _OPENMP
   if (threads <= 0) threads = omp_get_max_threads();
 #else
@@ -500,7 +555,7 @@ ORACLE_API float oracle_normal_from_words(uint32_t w0, uint32_t w1) {
  *       1 = N(0,1)*scale      2 = U(-1,1)*scale      3 = integers {-1,0,1}
  *           (kind 3 mirrors intel/test/utils.hpp:35-41: uniform(-2,2)
  *            truncated toward zero, so every partial sum is exact)
- * dtype: 0 = int8, 1 = bf16, 2 = fp16, 3 = fp32, 4 = int32                  */
+ * dtype: 0 = int8, 1 = bf16, 2 = fp16, 3 = fp32, 4 = int32, 5 = fp8 e4m3, 6 = fp8 e5m2 (saturating) */
 static float fill_value(int kind, float scale, uint64_t seed, uint64_t idx) {
   uint32_t w[4];
   philox_elem(seed, idx, w);
@@ -514,7 +569,7 @@ static float fill_value(int kind, float scale, uint64_t seed, uint64_t idx) {
 
 ORACLE_API int oracle_fill(void* dst, int64_t count, int dtype, int kind, float scale, uint64_t seed,
                            int threads) {
-  if (count < 0 || dtype < 0 || dtype > 4 || kind < 0 || kind > 3) return 1;
+  if (count < 0 || dtype < 0 || dtype > 6 || kind < 0 || kind > 3) return 1;
 #ifdef _OPENMP
   if (threads <= 0) threads = omp_get_max_threads();
 #else
@@ -524,6 +579,8 @@ ORACLE_API int oracle_fill(void* dst, int64_t count, int dtype, int kind, float 
   for (int64_t i = 0; i < count; i++) {
     float v = fill_value(kind, scale, seed, (uint64_t)i);
     switch (dtype) {
+      case 5: ((uint8_t*)dst)[i] = oracle_f32_to_fp8(0, v); break;
+      case 6: ((uint8_t*)dst)[i] = oracle_f32_to_fp8(1, v); break;
       case 0: ((int8_t*)dst)[i] = (int8_t)v; break;
       case 1: ((uint16_t*)dst)[i] = oracle_f32_to_bf16(v); break;
       case 2: ((uint16_t*)dst)[i] = oracle_f32_to_f16(v); break;

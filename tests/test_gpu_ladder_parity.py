@@ -10,7 +10,7 @@ import oracle_lib as O
 pytestmark = pytest.mark.gpu
 
 LAYOUTS = list(itertools.product((O.ROW, O.COL), repeat=2))
-ALL_TYPES = (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32)
+ALL_TYPES = (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32, O.E4M3E4M3F16, O.E5M2E5M2F16)
 SKINNY_TYPES = (O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16)
 VALU_RUNGS = (0, 1, 2, 3)
 MFMA = 4
@@ -98,7 +98,8 @@ def test_skinny_rung(G, types):
 
 def test_skinny_rung_refuses_what_it_cannot_do(G):
     a = torch.zeros(129 * 64, dtype=torch.int16, device="cuda")
-    for kw in (dict(m=129), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32), dict(types=O.F32F32F32)):
+    for kw in (dict(m=129), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32), dict(types=O.F32F32F32),
+               dict(types=O.E4M3E4M3F16)):
         args = dict(types=O.BF16BF16BF16, m=8, n=64, k=64, la=O.ROW, lb=O.COL)
         args.update(kw)
         with pytest.raises(G.capi.GzError) as e:

@@ -23,7 +23,7 @@ def test_functor_instantiation_follows_the_reference_names(F, capi):
     assert F.functor("tf32_mma_gemm", "f32", "f32", 128, 128, 32).types == capi.F32F32F32
     assert F.functor("naive_gemm", "f32", "f32")(128, 128, 128).plan.rung == capi.RUNG_NAIVE
     with pytest.raises(KeyError):
-        F.functor("fp8_mma_gemm", "f32", "f32")        # no such functor
+        F.functor("fp4_mma_gemm", "f32", "f32")        # no such functor
     with pytest.raises(KeyError):
         F.functor("naive_gemm", "bf16", "s32")
 
