@@ -65,7 +65,7 @@ const char* gz_hipblaslt_last_error(void) { return g_err; }
 
 // Plans D(MxN, row-major) = alpha * A x B + beta * C for one type bundle and layout pair.
 int gz_hipblaslt_create(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, void** plan_out) {
-  if (!plan_out || types < 0 || types > GZ_F32F32F32 || M <= 0 || N <= 0 || K <= 0 || (layoutA | layoutB) & ~1) {
+  if (!plan_out || types < 0 || types >= GZ_NUM_TYPES || M <= 0 || N <= 0 || K <= 0 || (layoutA | layoutB) & ~1) {
     set_err("gz_hipblaslt_create: bad argument");
     return GZ_ERR_BAD_ARG;
   }
@@ -75,6 +75,8 @@ int gz_hipblaslt_create(int types, int64_t M, int64_t N, int64_t K, int layoutA,
     case GZ_S8S8S32: in_t = HIP_R_8I; out_t = HIP_R_32I; scale_t = HIP_R_32I; comp = HIPBLAS_COMPUTE_32I; break;
     case GZ_BF16BF16F32: in_t = HIP_R_16BF; out_t = HIP_R_32F; scale_t = HIP_R_32F; comp = HIPBLAS_COMPUTE_32F; break;
     case GZ_BF16BF16BF16: in_t = HIP_R_16BF; out_t = HIP_R_16BF; scale_t = HIP_R_32F; comp = HIPBLAS_COMPUTE_32F; break;
+    case GZ_E4M3E4M3F16: in_t = HIP_R_8F_E4M3; out_t = HIP_R_16F; scale_t = HIP_R_32F; comp = HIPBLAS_COMPUTE_32F; break;
+    case GZ_E5M2E5M2F16: in_t = HIP_R_8F_E5M2; out_t = HIP_R_16F; scale_t = HIP_R_32F; comp = HIPBLAS_COMPUTE_32F; break;
     case GZ_F32F32F32: in_t = HIP_R_32F; out_t = HIP_R_32F; scale_t = HIP_R_32F; comp = HIPBLAS_COMPUTE_32F; break;
     default: in_t = HIP_R_16F; out_t = HIP_R_16F; scale_t = HIP_R_32F; comp = HIPBLAS_COMPUTE_32F; break;
   }

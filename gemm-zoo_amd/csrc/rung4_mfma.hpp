@@ -699,6 +699,20 @@ __device__ __forceinline__ void asm_mfma32(typename AccVec<TYPES>::type& c, cons
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
 }
 
+// v_mfma_f32_32x32x64_f8f6f4 on 8-bit floats: 32 bytes per lane and operand, given as the fragments of two
+// consecutive 32-byte K steps (cbsz / blgp select the format of the two operands: 0 e4m3, 1 e5m2)
+typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
+template <int TYPES>
+__device__ __forceinline__ void asm_mfma_f8(typename AccVec<TYPES>::type& c, const u32x4_t& first0, const u32x4_t& first1,
+                                            const u32x4_t& second0, const u32x4_t& second1) {
+  const u32x8_t f = __builtin_shufflevector(first0, first1, 0, 1, 2, 3, 4, 5, 6, 7);
+  const u32x8_t s = __builtin_shufflevector(second0, second1, 0, 1, 2, 3, 4, 5, 6, 7);
+  if constexpr (TYPES == GZ_E5M2E5M2F16)
+    asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(c) : "v"(f), "v"(s));
+  else
+    asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(f), "v"(s));
+}
+
 // orders later reads of an accumulator after every asm statement that precedes this one
 template <int TYPES> __device__ __forceinline__ void asm_touch_acc(typename AccVec<TYPES>::type& c) {
   asm volatile("" : "+a"(c));
@@ -937,11 +951,12 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   const bool edge = shape_class != MFMA_SHAPE_WHOLE;
   // the fixed instruction sequences are written for one MFMA per fragment pair; the 8-bit float types run the
   // compiler-scheduled direct-to-LDS kernel on whole tiles
-  constexpr bool HAND_SCHEDULED = !is_fp8(TYPES);
+  constexpr bool HAND_SCHEDULED = !is_fp8(TYPES);  // mfma_asm_kernel
+  constexpr bool PIPE4 = true;
   if constexpr (TYPES != GZ_F32F32F32) {  // fp32 runs the register-staged kernel only: its MFMAs are 8x longer per byte
   // M or N not a multiple of the tile, everything else in order: the hand-scheduled 256x256 kernels clamp rows
   if (shape_class == MFMA_SHAPE_RAGGED_MN && akc && hand_scheduled == 2) {
-    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+    if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
       const size_t plds = 4u * (size_t)(BM + BN) * 64;
       if (bkc) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>;
@@ -962,7 +977,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   }
   if (!edge && akc && bkc) {  // whole tiles, K-contiguous operands, aligned: direct-to-LDS fast path
     const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
-    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+    if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
         const size_t plds = 4u * (size_t)(BM + BN) * 64;
@@ -1000,7 +1015,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
       GZ_HIP_TRY(hipGetLastError());
       return GZ_OK;
     }
-    if constexpr (HAND_SCHEDULED && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
+    if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;
         const size_t plds = 4u * (size_t)(BM + BN) * 64;

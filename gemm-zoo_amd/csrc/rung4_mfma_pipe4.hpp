@@ -208,8 +208,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
   });
   asm volatile("s_nop 7" ::: "memory");
-  u32x4_t af[2][FM], bf[2][FN];
-  u32x2_t bh[2][FN][2];  // row-major B: the two halves of a fragment as they come out of the transposing reads
+  // Register sets of fragments: one per MFMA step.  The 8-bit float types use v_mfma_f32_32x32x64_f8f6f4, whose
+  // operands are the fragments of both steps of a half-slab side by side, so they keep four sets: set 2 P + ks holds
+  // step ks of the half-slabs of parity P.
+  constexpr bool F8 = is_fp8(TYPES);
+  constexpr int NSETS = F8 ? 4 : 2;
+  u32x4_t af[NSETS][FM], bf[NSETS][FN];
+  u32x2_t bh[NSETS][FN][2];  // row-major B: the two halves of a fragment as they come out of the transposing reads
 
   auto read_one = [&](auto set_c, auto r_c, int st, int ks) {
     constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value;
@@ -254,6 +259,44 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     });
   };
 
+  // 8-bit floats: half a half-slab's MFMAs (each covers both K steps: 64 K values, 16 passes) on the sets of parity P;
+  // meanwhile the fragments of (buffer rst, step PART) go to the sets of the other parity and this part's copies are
+  // issued, up to two memory instructions after each MFMA.  The fragments were waited for at the barrier.
+  auto step_f8 = [&](auto p_c, auto part_c, int rst, auto copy_is_a, int cst, int chs, uint64_t cmask) {
+    constexpr int P = decltype(p_c)::value, PART = decltype(part_c)::value;
+    constexpr bool IS_A = decltype(copy_is_a)::value;
+    constexpr int NC = IS_A ? A_PW : B_PW;
+    constexpr int NOPS = NRD + NC, HALF_MMA = NMMA / 2;
+    constexpr int PER = (NOPS + HALF_MMA - 1) / HALF_MMA;
+    static_assert(PER <= 2, "at most two memory instructions per MFMA");
+    if constexpr (PART == 0 && !B_KC) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+          asm volatile("" : "+v"(bh[2 * P + ks][j][0]), "+v"(bh[2 * P + ks][j][1]));  // after the wait
+          bf[2 * P + ks][j] = u32x4_t{bh[2 * P + ks][j][0][0], bh[2 * P + ks][j][0][1], bh[2 * P + ks][j][1][0],
+                                      bh[2 * P + ks][j][1][1]};
+        }
+    }
+    if constexpr (IS_A) copy_a_begin(cst);
+    else copy_b_begin(cst);
+    static_for<HALF_MMA>([&](auto q_c) {
+      constexpr int QL = decltype(q_c)::value, Q = PART * HALF_MMA + QL;
+      asm_mfma_f8<TYPES>(acc[Q / FN][Q % FN], bf[2 * P][Q % FN], bf[2 * P + 1][Q % FN], af[2 * P][Q / FN],
+                         af[2 * P + 1][Q / FN]);
+      static_for<PER>([&](auto o_c) {
+        constexpr int OP = QL * PER + decltype(o_c)::value;
+        if constexpr (OP < NRD) {
+          read_one(std::integral_constant<int, 2 * (P ^ 1) + PART>{}, std::integral_constant<int, OP>{}, rst, PART);
+        } else if constexpr (OP < NOPS) {
+          if constexpr (IS_A) copy_a(std::integral_constant<int, OP - NRD>{}, chs, cmask);
+          else copy_b(std::integral_constant<int, OP - NRD>{}, chs, cmask);
+        }
+      });
+    });
+  };
+
   const std::true_type is_a{};
   const std::false_type is_b{};
   using I0 = std::integral_constant<int, 0>;
@@ -277,21 +320,40 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   {
     const uint64_t m3 = mask_if(3 < nh);
     static_for<A_PW>([&](auto t) { copy_a(t, 3, m3); });
+    if constexpr (F8) {  // the 8-bit float pipeline runs half a half-slab earlier: all of half-slab 3 here
+      copy_b_begin(3);
+      static_for<B_PW>([&](auto t) { copy_b(t, 3, m3); });
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");  // simple and safe: the prologue is short
   static_for<NRD>([&](auto r) { read_one(I0{}, r, 0, 0); });
+  if constexpr (F8) static_for<NRD>([&](auto r) { read_one(I1{}, r, 0, 1); });
 
   // ---- one half-slab; S = h % 4 at compile time ----
   auto half_slab = [&](auto s_c, int h) {
     constexpr int S = decltype(s_c)::value;
-    step(I0{}, S, 1, is_b, (S + 3) % NST, h + 3, mask_if(h + 3 < nh));
-    if (h + 3 < nh) {  // the 2 * NCP copies issued after those of half-slab h+1 may stay in flight
-      if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (F8) {
+      // barrier first: this wave has the fragments of half-slab h (both steps), so buffer S is free once every wave
+      // is here, and its copies of half-slab h+1 have landed (the 2 * NCP issued after them may stay in flight)
+      if (h + 3 < nh) {
+        if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      }
+      const uint64_t m4 = mask_if(h + 4 < nh);
+      step_f8(std::integral_constant<int, S & 1>{}, I0{}, (S + 1) % NST, is_b, S, h + 4, m4);
+      step_f8(std::integral_constant<int, S & 1>{}, I1{}, (S + 1) % NST, is_a, S, h + 4, m4);
     } else {
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      step(I0{}, S, 1, is_b, (S + 3) % NST, h + 3, mask_if(h + 3 < nh));
+      if (h + 3 < nh) {  // the 2 * NCP copies issued after those of half-slab h+1 may stay in flight
+        if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      }
+      step(I1{}, (S + 1) % NST, 0, is_a, S, h + 4, mask_if(h + 4 < nh));
     }
-    step(I1{}, (S + 1) % NST, 0, is_a, S, h + 4, mask_if(h + 4 < nh));
   };
 
   for (int h = 0; h < nh; h += 4) {

@@ -48,6 +48,8 @@ template <> struct elem<gemm_zoo::bf16_t> { static constexpr int dt = 1, kind = 
 template <> struct elem<gemm_zoo::half_t> { static constexpr int dt = 2, kind = 1; };
 template <> struct elem<float> { static constexpr int dt = 3, kind = 1; };
 template <> struct elem<int32_t> { static constexpr int dt = 4, kind = 0; };
+template <> struct elem<gemm_zoo::e4m3_t> { static constexpr int dt = 5, kind = 1; };
+template <> struct elem<gemm_zoo::e5m2_t> { static constexpr int dt = 6, kind = 1; };
 
 struct result {
   double mean_ms, median_ms, gflops_ref, tflops, gbps;

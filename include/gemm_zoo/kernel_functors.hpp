@@ -30,6 +30,9 @@ namespace gemm_zoo {
 // 16-bit storage types (bit patterns); enough for hosts that only move data around.
 struct bf16_t { uint16_t bits; };
 struct half_t { uint16_t bits; };
+// OCP 8-bit floats (the formats of __nv_fp8_e4m3 / __nv_fp8_e5m2), inputs only
+struct e4m3_t { uint8_t bits; };
+struct e5m2_t { uint8_t bits; };
 
 enum class layout : int { row_major = GZ_ROW_MAJOR, col_major = GZ_COL_MAJOR };
 
@@ -48,6 +51,9 @@ template <> struct bundle<bf16_t, float> { static constexpr int value = GZ_BF16B
 template <> struct bundle<bf16_t, bf16_t> { static constexpr int value = GZ_BF16BF16BF16; };
 template <> struct bundle<half_t, half_t> { static constexpr int value = GZ_F16F16F16; };
 template <> struct bundle<float, float> { static constexpr int value = GZ_F32F32F32; };  // the reference's ladder drivers
+// nvidia/bench/bench_cublaslt_e4m3.cu:9-11, bench_cublaslt_e5m2.cu:9-11
+template <> struct bundle<e4m3_t, half_t> { static constexpr int value = GZ_E4M3E4M3F16; };
+template <> struct bundle<e5m2_t, half_t> { static constexpr int value = GZ_E5M2E5M2F16; };
 
 template <typename TIn, typename TOut, layout LA, layout LB> class functor_base {
  public:
@@ -163,6 +169,16 @@ struct tf32_mma_gemm : detail::functor_base<TIn, TOut, LA, LB> {
 template <typename TIn, typename TOut, int M = 128, int N = 128, int K = 32, layout LA = layout::row_major,
           layout LB = layout::row_major>
 using f32_mma_gemm = tf32_mma_gemm<TIn, TOut, M, N, K, LA, LB>;
+
+// fp8 x fp8 -> fp16 on the matrix cores; no counterpart in the reference, which runs these types through cuBLASLt
+// only (nvidia/bench/bench_cublaslt_e4m3.cu, bench_cublaslt_e5m2.cu)
+template <typename TIn, typename TOut, int M = 256, int N = 256, int K = 128, layout LA = layout::row_major,
+          layout LB = layout::row_major>
+struct fp8_mma_gemm : detail::functor_base<TIn, TOut, LA, LB> {
+  static_assert((std::is_same_v<TIn, e4m3_t> || std::is_same_v<TIn, e5m2_t>) && std::is_same_v<TOut, half_t>,
+                "fp8 in, fp16 out");
+  GZ_FUNCTOR_COMMON(fp8_mma_gemm, GZ_RUNG_MFMA, detail::mfma_variant_for(M, N))
+};
 
 // int8 x int8 -> int32 on the matrix cores
 template <typename TIn, typename TOut, int M = 256, int N = 256, int K = 128, layout LA = layout::row_major,
