@@ -24,7 +24,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
-PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0}  # dense MFMA, MI355X
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "fp8": 5000.0}  # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 INFINITY_CACHE_BYTES = 256 * 1000 * 1000
 
@@ -60,13 +60,13 @@ def main() -> int:
     sptr = stream.cuda_stream
 
     IN_T = {capi.S8S8S32: torch.int8, capi.BF16BF16F32: torch.bfloat16, capi.BF16BF16BF16: torch.bfloat16,
-            capi.F16F16F16: torch.float16}
+            capi.F16F16F16: torch.float16, capi.E4M3E4M3F16: torch.float8_e4m3fn, capi.E5M2E5M2F16: torch.float8_e5m2}
     OUT_T = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
-             capi.F16F16F16: torch.float16}
+             capi.F16F16F16: torch.float16, capi.E4M3E4M3F16: torch.float16, capi.E5M2E5M2F16: torch.float16}
     OUT_DT = {capi.S8S8S32: capi.DT_INT32, capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16,
-              capi.F16F16F16: capi.DT_F16}
+              capi.F16F16F16: capi.DT_F16, capi.E4M3E4M3F16: capi.DT_F16, capi.E5M2E5M2F16: capi.DT_F16}
     IN_DT = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
-             capi.F16F16F16: capi.DT_F16}
+             capi.F16F16F16: capi.DT_F16, capi.E4M3E4M3F16: capi.DT_E4M3, capi.E5M2E5M2F16: capi.DT_E5M2}
 
     def make_sets(types, m, n, k, scale_b=1.0, seed0=2025):
         """P rotating (A, B) sets + one D, filled on the device (seeds 2025, 2026, ... as the reference harness)."""
@@ -110,7 +110,7 @@ def main() -> int:
             if types == capi.S8S8S32:
                 ndiff = capi.compare(d, ref, m * n, capi.DT_INT32, 0.0, sptr)
             else:
-                dt = {capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16, capi.F16F16F16: capi.DT_F16}[types]
+                dt = OUT_DT[types]
                 # sanity bound only (parity proper lives in tests/): fp32 accumulation in a different order, so allow
                 # 1e-3 of the output scale for fp32 out and one 16-bit ulp at 4 sigma for 16-bit out
                 scale = float(torch.sqrt(torch.tensor(float(k)))) * scale_b
@@ -193,13 +193,22 @@ def main() -> int:
         rr = timed(capi.BF16BF16F32, M, N, K, capi.ROW_MAJOR, capi.ROW_MAJOR, args.steps, args.warmup)
         extras["bf16_4096_row_row"] = {"tflops": round(flops / (rr["kernel_ms_mean"] * 1e-3) / 1e12, 2),
                                        "kernel_ms_mean": round(rr["kernel_ms_mean"], 5)}
+        # next row of the scope: fp8 e4m3 x e4m3 -> fp16 (the reference times cuBLASLt on it,
+        # nvidia/bench/bench_cublaslt_e4m3.cu:6-21), this library's own kernel on the reference drivers' layout
+        # (row-major A and B); inputs N(0, 0.25) so that the fp16 outputs of K = 8192 stay far from overflow
+        rf = timed(capi.E4M3E4M3F16, m8, m8, m8, capi.ROW_MAJOR, capi.ROW_MAJOR, 30, 40, scale_b=0.25)
+        tf8 = 2.0 * m8 ** 3 / (rf["kernel_ms_mean"] * 1e-3) / 1e12
+        extras["e4m3_8192_row_row"] = {"tflops": round(tf8, 2), "frac_of_fp8_peak": round(tf8 / PEAK_TFLOPS["fp8"], 4),
+                                       "kernel_ms_mean": round(rf["kernel_ms_mean"], 5)}
         # the vendor library beside it (the reference reports cuBLASLt): same operands, same timing, checked the same way
         try:
             functors = importlib.import_module("gemm-zoo_amd.functors")
-            for name, (ty, sz, st, wu) in {"hipblaslt_bf16_4096": (capi.BF16BF16F32, 4096, args.steps, args.warmup),
-                                           "hipblaslt_s8_8192": (capi.S8S8S32, 8192, 30, 40)}.items():
-                lt = functors.HipblasLtGemm(ty, sz, sz, sz, capi.ROW_MAJOR, capi.COL_MAJOR)
-                rl = timed(ty, sz, sz, sz, capi.ROW_MAJOR, capi.COL_MAJOR, st, wu, vendor=lt)
+            for name, (ty, sz, st, wu, lb, sb) in {
+                    "hipblaslt_bf16_4096": (capi.BF16BF16F32, 4096, args.steps, args.warmup, capi.COL_MAJOR, 1.0),
+                    "hipblaslt_s8_8192": (capi.S8S8S32, 8192, 30, 40, capi.COL_MAJOR, 1.0),
+                    "hipblaslt_e4m3_8192_row_row": (capi.E4M3E4M3F16, 8192, 30, 40, capi.ROW_MAJOR, 0.25)}.items():
+                lt = functors.HipblasLtGemm(ty, sz, sz, sz, capi.ROW_MAJOR, lb)
+                rl = timed(ty, sz, sz, sz, capi.ROW_MAJOR, lb, st, wu, vendor=lt, scale_b=sb)
                 extras[name] = {"tflops": round(2.0 * sz ** 3 / (rl["kernel_ms_mean"] * 1e-3) / 1e12, 2),
                                 "kernel_ms_mean": round(rl["kernel_ms_mean"], 5)}
                 lt.close()

@@ -212,7 +212,10 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // operands are the fragments of both steps of a half-slab side by side, so they keep four sets: set 2 P + ks holds
   // step ks of the half-slabs of parity P.
   constexpr bool F8 = is_fp8(TYPES);
-  constexpr int NSETS = F8 ? 4 : 2;
+  // (The same half-slab-ahead schedule works for the other types, one step's MFMAs per part; measured against
+  // hipBLASLt in the same run it changed bf16 4096^3 by -1 % and int8 8192^3 by +2 %, so they keep two sets.)
+  constexpr bool DEEP = F8;
+  constexpr int NSETS = DEEP ? 4 : 2;
   u32x4_t af[NSETS][FM], bf[NSETS][FN];
   u32x2_t bh[NSETS][FN][2];  // row-major B: the two halves of a fragment as they come out of the transposing reads
 
@@ -266,12 +269,12 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     constexpr int P = decltype(p_c)::value, PART = decltype(part_c)::value;
     constexpr bool IS_A = decltype(copy_is_a)::value;
     constexpr int NC = IS_A ? A_PW : B_PW;
-    constexpr int NOPS = NRD + NC, HALF_MMA = NMMA / 2;
-    constexpr int PER = (NOPS + HALF_MMA - 1) / HALF_MMA;
+    constexpr int NOPS = NRD + NC, PART_MMA = F8 ? NMMA / 2 : NMMA;
+    constexpr int PER = (NOPS + PART_MMA - 1) / PART_MMA;
     static_assert(PER <= 2, "at most two memory instructions per MFMA");
-    if constexpr (PART == 0 && !B_KC) {
+    if constexpr (!B_KC && (PART == 0 || !F8)) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++)
+      for (int ks = F8 ? 0 : PART; ks < (F8 ? 2 : PART + 1); ks++)
 #pragma unroll
         for (int j = 0; j < FN; j++) {
           asm volatile("" : "+v"(bh[2 * P + ks][j][0]), "+v"(bh[2 * P + ks][j][1]));  // after the wait
@@ -281,10 +284,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     }
     if constexpr (IS_A) copy_a_begin(cst);
     else copy_b_begin(cst);
-    static_for<HALF_MMA>([&](auto q_c) {
-      constexpr int QL = decltype(q_c)::value, Q = PART * HALF_MMA + QL;
-      asm_mfma_f8<TYPES>(acc[Q / FN][Q % FN], bf[2 * P][Q % FN], bf[2 * P + 1][Q % FN], af[2 * P][Q / FN],
-                         af[2 * P + 1][Q / FN]);
+    static_for<PART_MMA>([&](auto q_c) {
+      constexpr int QL = decltype(q_c)::value, Q = F8 ? PART * PART_MMA + QL : QL;
+      if constexpr (F8)
+        asm_mfma_f8<TYPES>(acc[Q / FN][Q % FN], bf[2 * P][Q % FN], bf[2 * P + 1][Q % FN], af[2 * P][Q / FN],
+                           af[2 * P + 1][Q / FN]);
+      else
+        asm_mfma32<TYPES>(acc[Q / FN][Q % FN], bf[2 * P + PART][Q % FN], af[2 * P + PART][Q / FN]);
       static_for<PER>([&](auto o_c) {
         constexpr int OP = QL * PER + decltype(o_c)::value;
         if constexpr (OP < NRD) {
@@ -320,19 +326,19 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   {
     const uint64_t m3 = mask_if(3 < nh);
     static_for<A_PW>([&](auto t) { copy_a(t, 3, m3); });
-    if constexpr (F8) {  // the 8-bit float pipeline runs half a half-slab earlier: all of half-slab 3 here
+    if constexpr (DEEP) {  // the 8-bit float pipeline runs half a half-slab earlier: all of half-slab 3 here
       copy_b_begin(3);
       static_for<B_PW>([&](auto t) { copy_b(t, 3, m3); });
     }
   }
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");  // simple and safe: the prologue is short
   static_for<NRD>([&](auto r) { read_one(I0{}, r, 0, 0); });
-  if constexpr (F8) static_for<NRD>([&](auto r) { read_one(I1{}, r, 0, 1); });
+  if constexpr (DEEP) static_for<NRD>([&](auto r) { read_one(I1{}, r, 0, 1); });
 
   // ---- one half-slab; S = h % 4 at compile time ----
   auto half_slab = [&](auto s_c, int h) {
     constexpr int S = decltype(s_c)::value;
-    if constexpr (F8) {
+    if constexpr (DEEP) {
       // barrier first: this wave has the fragments of half-slab h (both steps), so buffer S is free once every wave
       // is here, and its copies of half-slab h+1 have landed (the 2 * NCP issued after them may stay in flight)
       if (h + 3 < nh) {

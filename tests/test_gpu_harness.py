@@ -16,7 +16,8 @@ def G():
     return gpu_util
 
 
-@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32])
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32,
+                                   O.E4M3E4M3F16, O.E5M2E5M2F16])
 def test_hipblaslt_comparator_against_oracle(G, types):
     """The comparator is only trusted after it has itself been checked: every layout pair, exact on integer data."""
     import torch
@@ -52,6 +53,10 @@ def test_harness_runs_verifies_and_reports(G, capsys):
     # the reference's fp32 drivers: LDS rung and the matrix-core functor that stands in for tf32_mma_gemm
     for name in ("smem_tiled_gemm", "tf32_mma_gemm"):
         r = H.benchmark(F.functor(name, "f32", "f32", 128, 128, 32), [(384, 256, 160)], 1.0, 1.0, num_repititions=2)[0]
+        assert r.tflops > 0
+    # fp8 in, fp16 out (the bundles of nvidia/bench/bench_cublaslt_e4m3.cu / _e5m2.cu) on this library's own kernels
+    for tin in ("e4m3", "e5m2"):
+        r = H.benchmark(F.functor("fp8_mma_gemm", tin, "f16"), [(512, 256, 384)], 1.0, 1.0, num_repititions=2)[0]
         assert r.tflops > 0
     S = F.functor("gemm_s8_s8_s32_m8k16", "s8", "s32", layout_b=F.COL)
     r = H.benchmark_sizes(S, [(512, 512, 512)], num_repititions=2)[0]
