@@ -8,7 +8,7 @@ import oracle_lib as O
 pytestmark = pytest.mark.gpu
 
 TORCH_OF_DT = {O.DT_INT8: torch.int8, O.DT_BF16: torch.int16, O.DT_F16: torch.int16, O.DT_F32: torch.float32,
-               O.DT_INT32: torch.int32}
+               O.DT_INT32: torch.int32, O.DT_E4M3: torch.uint8, O.DT_E5M2: torch.uint8}
 
 
 @pytest.fixture(scope="module")
@@ -17,12 +17,15 @@ def G():
     return gpu_util
 
 
-@pytest.mark.parametrize("dtype", [O.DT_INT8, O.DT_BF16, O.DT_F16, O.DT_F32, O.DT_INT32])
+@pytest.mark.parametrize("dtype", [O.DT_INT8, O.DT_BF16, O.DT_F16, O.DT_F32, O.DT_INT32, O.DT_E4M3, O.DT_E5M2])
 @pytest.mark.parametrize("kind", [O.FILL_INT8_UNIFORM, O.FILL_NORMAL, O.FILL_UNIFORM_PM1, O.FILL_SMALL_INT])
 def test_device_fill_matches_cpu_fill_bit_for_bit(G, dtype, kind):
     if dtype in (O.DT_INT8, O.DT_INT32) and kind in (O.FILL_NORMAL, O.FILL_UNIFORM_PM1):
         pytest.skip("real-valued kinds are for float destinations")
-    for count, seed, scale in [(1, 1, 1.0), (1000003, 2025, 1.0), (70000, (5 << 32) | 17, 0.02)]:
+    cases = [(1, 1, 1.0), (1000003, 2025, 1.0), (70000, (5 << 32) | 17, 0.02)]
+    if dtype in (O.DT_E4M3, O.DT_E5M2):  # 8-bit floats: also the subnormal range and saturation at the top
+        cases += [(50000, 3, 2.0 ** -8), (50000, 4, 2.0 ** -15), (50000, 5, 300.0), (50000, 6, 1e6)]
+    for count, seed, scale in cases:
         t = torch.zeros(count + 8, dtype=TORCH_OF_DT[dtype], device="cuda")
         G.capi.fill(t, count, dtype, kind, scale, seed, torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
