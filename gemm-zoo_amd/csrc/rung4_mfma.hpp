@@ -53,6 +53,7 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, first),
                                                   __builtin_bit_cast(f16x8_t, second), acc, 0, 0, 0);
   } else if constexpr (is_fp8(TYPES)) {
+    // One fragment pair alone (the kernels' own loops for these types pair two K steps instead, see mfma_f8_pair):
     // 16 bytes per lane are 16 K values; v_mfma_f32_32x32x16_{fp8_fp8,bf8_bf8} takes 8 per lane, so the two halves
     // of the fragment pair feed one instruction each (which k a lane's bytes stand for is the same on both
     // operands, and that is all a dot product needs).
@@ -83,6 +84,18 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
 
 // MFMA instructions behind one mfma32 call
 template <int TYPES> constexpr int mfmas_per_fragment() { return TYPES == GZ_F32F32F32 ? 4 : is_fp8(TYPES) ? 2 : 1; }
+
+// 8-bit floats, the fragments of two consecutive 32-byte K steps at once: v_mfma_f32_32x32x64_f8f6f4 takes 32 bytes
+// per lane and operand (format 0 = e4m3, 1 = e5m2; no block scaling).  Which k a lane's bytes stand for is the same
+// on both operands.
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+template <int TYPES>
+__device__ inline f32x16_t mfma_f8_pair(u32x4_t first0, u32x4_t first1, u32x4_t second0, u32x4_t second1, f32x16_t acc) {
+  const i32x8_t f = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(first0, first1, 0, 1, 2, 3, 4, 5, 6, 7));
+  const i32x8_t s = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(second0, second1, 0, 1, 2, 3, 4, 5, 6, 7));
+  constexpr int FMT = TYPES == GZ_E5M2E5M2F16 ? 1 : 0;
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f, s, acc, FMT, FMT, 0, 0, 0, 0);
+}
 
 constexpr int SLAB_BYTES = 128;           // K bytes per tile row per slab
 constexpr int PITCH = SLAB_BYTES + 16;    // LDS row pitch
@@ -130,6 +143,17 @@ template <int MASK, int N_OTHER, int N_MFMA> __device__ inline void mix_into_mfm
       __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
       __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
     }
+  }
+}
+
+// The same for two classes at once: N_ST LDS stores, then N_LD global loads, after each MFMA its share of both.
+template <int N_ST, int N_LD, int N_MFMA> __device__ inline void mix2_into_mfmas() {
+  constexpr int PER_ST = (N_ST + N_MFMA - 1) / N_MFMA, PER_LD = (N_LD + N_MFMA - 1) / N_MFMA;
+#pragma unroll
+  for (int x = 0; x < N_MFMA; x++) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x200, PER_ST, 0);
+    __builtin_amdgcn_sched_group_barrier(0x020, PER_LD, 0);
   }
 }
 
@@ -318,8 +342,10 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   const int b_off = A_BYTES + (B_NAT ? (lane >> 5) * 4 * StagerB::NAT_PITCH + (wn * WN + frag_row) * 4
                                      : (wn * WN + frag_row) * PITCH + frag_k);
 
-  // Two fragment sets: while the MFMAs of one K step run, the ds_reads of the next are in flight.
-  u32x4_t af[2][FM], bf[2][FN];
+  // Two fragment sets: while the MFMAs of one K step run, the ds_reads of the next are in flight.  (8-bit floats:
+  // two pairs of sets, a pair holds two consecutive K steps for one 64-deep MFMA.)
+  constexpr bool F8 = is_fp8(TYPES);
+  u32x4_t af[F8 ? 4 : 2][FM], bf[F8 ? 4 : 2][FN];
   auto read_frags = [&](int set, const char* stage, int ks) {
 #pragma unroll
     for (int i = 0; i < FM; i++) {
@@ -378,6 +404,37 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // and what is parked in LDS then is never read.
   static_assert(KSTEPS == 4, "the slab loop is written out for four steps");
   constexpr int MFMAS_PER_STEP = FM * FN * mfmas_per_fragment<TYPES>();
+  if constexpr (F8) {
+    // 8-bit floats: the same loop in two double steps, each one v_mfma_f32_32x32x64_f8f6f4 per 32x32 block
+    auto mma2 = [&](int pair) {
+#pragma unroll
+      for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+          acc[i][j] = mfma_f8_pair<TYPES>(bf[2 * pair][j], bf[2 * pair + 1][j], af[2 * pair][i], af[2 * pair + 1][i], acc[i][j]);
+    };
+    read_frags(1, lds, 1);
+    for (int kt = 0; kt < ktiles; kt++) {
+      const char* cur = lds + (kt & 1) * STAGE_BYTES;
+      char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+      read_frags(2, cur, 2);
+      read_frags(3, cur, 3);
+      sa.store(nxt, tid);
+      sb.store(nxt + A_BYTES, tid);
+      const int k_next = (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK;
+      sa.load(g.A, g.M, g.K, m0, k_next, tid);
+      sb.load(g.B, g.N, g.K, n0, k_next, tid);
+      mma2(0);
+      mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, FM * FN>();
+      __builtin_amdgcn_sched_barrier(0);
+
+      __syncthreads();
+      read_frags(0, nxt, 0);
+      read_frags(1, nxt, 1);
+      mma2(1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else
   for (int kt = 0; kt < ktiles; kt++) {
     const char* cur = lds + (kt & 1) * STAGE_BYTES;
     char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
@@ -385,16 +442,15 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     read_frags(1, cur, 1);
     sa.store(nxt, tid);
     sb.store(nxt + A_BYTES, tid);
-    mma(0);
-    mix_into_mfmas<0x200, StagerA::LDS_STORES + StagerB::LDS_STORES, MFMAS_PER_STEP>();
-    __builtin_amdgcn_sched_barrier(0);
-
-    read_frags(0, cur, 2);
     const int k_next = (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK;
     sa.load(g.A, g.M, g.K, m0, k_next, tid);
     sb.load(g.B, g.N, g.K, n0, k_next, tid);
+    mma(0);
+    mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, MFMAS_PER_STEP>();
+    __builtin_amdgcn_sched_barrier(0);
+
+    read_frags(0, cur, 2);
     mma(1);
-    mix_into_mfmas<0x020, StagerA::VECS + StagerB::VECS, MFMAS_PER_STEP>();
     __builtin_amdgcn_sched_barrier(0);
 
     read_frags(1, cur, 3);
@@ -575,7 +631,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       tr_off[j] = A_BYTES + krow * TR_PITCH + (((n_local / EPV) ^ dtl_tr_swz<ES, PPR>(fi)) * 16) + (n_local % EPV) * ES;
     }
   }
-  u32x4_t af[2][FM], bf[2][FN];
+  constexpr bool F8 = is_fp8(TYPES);  // two pairs of fragment sets, a pair feeds one 64-deep MFMA per block
+  u32x4_t af[F8 ? 4 : 2][FM], bf[F8 ? 4 : 2][FN];
   auto read_frags = [&](int set, const char* stage, int ks) {
 #pragma unroll
     for (int i = 0; i < FM; i++)
@@ -609,6 +666,33 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // One barrier per slab.  At the barrier of slab kt every wave has finished reading buffer kt&1 and the
   // copies of slab kt+1 have landed, so the copies of slab kt+2 may overwrite buffer kt&1 right after it;
   // they then have a whole slab of MFMAs to complete.
+  if constexpr (F8) {
+    auto mma2 = [&](int pair) {
+#pragma unroll
+      for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+          acc[i][j] = mfma_f8_pair<TYPES>(bf[2 * pair][j], bf[2 * pair + 1][j], af[2 * pair][i], af[2 * pair + 1][i], acc[i][j]);
+    };
+    read_frags(1, lds, 1);
+    for (int kt = 0; kt < ktiles; kt++) {
+      char* cur = lds + (kt & 1) * STAGE_BYTES;
+      char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+      read_frags(2, cur, 2);
+      read_frags(3, cur, 3);
+      mma2(0);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+      __syncthreads();
+      if (kt + 2 < ktiles) copy_slab(cur, (kt + 2) * BK);
+      if (kt + 1 < ktiles) {
+        read_frags(0, nxt, 0);
+        read_frags(1, nxt, 1);
+      }
+      mma2(1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else
   for (int kt = 0; kt < ktiles; kt++) {
     char* cur = lds + (kt & 1) * STAGE_BYTES;
     char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
