@@ -184,10 +184,16 @@ __device__ inline typename Traits<TYPES>::out_t epilogue(typename Traits<TYPES>:
     }
     return f32_to_bf16(v);
   } else {
+    // The products pass through an empty asm statement before they are rounded to fp16: otherwise the compiler
+    // merges multiply and conversion into v_fma_mixlo_f16 with a +0 addend, which turns a product of -0 into +0.
     float v = round_out<TYPES>(acc);
-    v = round_out<TYPES>(mul_rn(v, alpha));
+    float p = mul_rn(v, alpha);
+    asm("" : "+v"(p));
+    v = round_out<TYPES>(p);
     if (beta != 0.0f) {
-      float bc = round_out<TYPES>(mul_rn(beta, f16_to_f32(*c_ptr)));
+      float q = mul_rn(beta, f16_to_f32(*c_ptr));
+      asm("" : "+v"(q));
+      const float bc = round_out<TYPES>(q);
       v = round_out<TYPES>(add_rn(v, bc));
     }
     return f32_to_f16(v);

@@ -152,3 +152,46 @@ def test_16bit_epilogue_rounding_order(G):
         assert O.bf16_to_f32(d)[0, 0] == 384.0
         d = G.run_gemm(O.BF16BF16BF16, bf([0.0]), bf([0.0]), bf([1.0078125]), 1, 1, 1, O.ROW, O.COL, 1.0, 1.0078125, rung)
         assert O.bf16_to_f32(d)[0, 0] == 1.015625
+
+
+@pytest.mark.parametrize("types", ALL_TYPES)
+def test_launcher_choice_on_random_problems(G, types):
+    """GZ_RUNG_AUTO on seeded random shapes, layouts and scalars (integer-valued data: bit-exact): whatever kernel
+    the launcher picks - streaming, direct-to-LDS, ragged, predicated - must give the oracle's bits."""
+    rng = np.random.default_rng(1000 + types)
+    es = np.dtype(O.IN_DTYPE[types]).itemsize
+    cases = []
+    for _ in range(14):
+        m, n, k = (int(rng.integers(1, 700)) for _ in range(3))
+        cases.append((m, n, k))
+    for _ in range(8):   # whole 16-byte rows and K slabs: the direct-to-LDS kernels, ragged or not
+        m, n = int(rng.integers(1, 5)) * 128 + int(rng.integers(0, 2)) * int(rng.integers(1, 128)), \
+            int(rng.integers(1, 5)) * 128 + int(rng.integers(0, 2)) * (16 // es) * int(rng.integers(1, 8))
+        cases.append((m, n, (128 // es) * int(rng.integers(1, 9))))
+    for _ in range(4):   # decode shapes
+        cases.append((int(rng.integers(1, 129)), int(rng.integers(1, 40)) * 16, 64 * int(rng.integers(1, 12))))
+    for m, n, k in cases:
+        la, lb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        al, be = int(rng.integers(-2, 3)), int(rng.integers(-1, 2))
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=m * 7 + n * 3 + k)
+        print("case", types, m, n, k, la, lb, al, be, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, al, be, G.capi.RUNG_AUTO)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, al, be)), (types, m, n, k, la, lb, al, be)
+
+
+@pytest.mark.parametrize("types", [O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32, O.E4M3E4M3F16])
+def test_sign_of_zero_survives_the_epilogue(G, types):
+    """alpha = 0 on negative sums and alpha < 0 on zero sums give -0 in IEEE arithmetic; a multiply fused with the
+    conversion to fp16 (fma with a +0 addend) would lose it."""
+    m, n, k = 64, 48, 40
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=5)
+    for (al, be), rung in itertools.product([(0, 0), (-2, 0), (0, 1), (-1, -1)], VALU_RUNGS + (MFMA,)):
+        ref = O.gemm(types, a, b, c, m, n, k, O.COL, O.ROW, al, be)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.COL, O.ROW, al, be, rung)
+        assert np.array_equal(got, ref), (types, al, be, rung)
+    # an all-zero product with a negative alpha
+    z = np.zeros_like(a)
+    ref = O.gemm(types, z, b, c, m, n, k, O.ROW, O.COL, -1, 0)
+    assert (ref.view(np.uint8).reshape(m * n, -1)[:, -1] == 0x80).all()
+    for rung in VALU_RUNGS + (MFMA,):
+        assert np.array_equal(G.run_gemm(types, z, b, c, m, n, k, O.ROW, O.COL, -1, 0, rung), ref), (types, rung)
