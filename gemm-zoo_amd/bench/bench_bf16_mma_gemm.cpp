@@ -1,5 +1,5 @@
 // Driver of nvidia/bench/bench_bf16_mma_gemm.cu:9-28 on the gfx950 ladder (same sizes, alpha = beta = 1),
-// followed by the BASELINE configuration (B column-major, beta = 0).
+// followed by the headline configuration of this library (B column-major, beta = 0).
 #include <tuple>
 
 #include "gemm_zoo/benchmark.hpp"

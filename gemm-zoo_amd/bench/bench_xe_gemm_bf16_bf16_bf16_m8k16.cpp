@@ -1,4 +1,4 @@
-// Driver of intel/bench/bench_xe_gemm_bf16_bf16_bf16_m8k16.cpp:10-19, plus the decode shapes of BASELINE
+// Driver of intel/bench/bench_xe_gemm_bf16_bf16_bf16_m8k16.cpp:10-19, plus the decode shapes
 // (weights column-major, reported in GB/s).
 #include <tuple>
 

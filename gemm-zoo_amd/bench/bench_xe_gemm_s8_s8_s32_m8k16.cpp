@@ -1,5 +1,5 @@
 // Driver of bench/bench_xe_gemm_s8_s8_s32_m8k16.cpp:10-18 (1024^3, 2048^3, 4096^3, alpha = beta = 1), plus the
-// BASELINE 8192^3 shape with column-major B.
+// 8192^3 shape with column-major B.
 #include <tuple>
 
 #include "gemm_zoo/benchmark.hpp"

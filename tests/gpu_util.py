@@ -10,7 +10,7 @@ import oracle_lib as O
 
 capi = importlib.import_module("gemm-zoo_amd.capi")
 
-TOL = {O.BF16BF16F32: 1e-3, O.BF16BF16BF16: 1e-2, O.F16F16F16: 1e-2,  # max relative error, BASELINE north_star
+TOL = {O.BF16BF16F32: 1e-3, O.BF16BF16BF16: 1e-2, O.F16F16F16: 1e-2,  # max relative error allowed for fp32 / 16-bit outputs
        O.F32F32F32: 1e-4,  # fp32 inputs: only the summation order differs
        O.E4M3E4M3F16: 1e-2, O.E5M2E5M2F16: 1e-2}  # fp16 output, exact products: the 16-bit-output bound
 

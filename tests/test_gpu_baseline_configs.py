@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their full sizes, through the C ABI.
+"""The five benchmark configurations (int8 1024^3 and 8192^3, bf16 4096^3, ragged fp16, decode shapes) at their full sizes, through the C ABI.
 
 Small ones are compared element for element with the CPU oracle.  The large ones (4096^3, 8192^3)
 are checked through size-independent properties that are exact for integers -- D x = A (B x) and
