@@ -50,6 +50,7 @@ class Plan(C.Structure):
         ("threads", C.c_int32), ("lds_bytes", C.c_int32),
         ("grid", C.c_int64), ("split_k", C.c_int32),
         ("vector_bytes_a", C.c_int32), ("vector_bytes_b", C.c_int32),
+        ("tail_rows", C.c_int32), ("tail_tile_m", C.c_int32), ("tail_tile_n", C.c_int32), ("tail_grid", C.c_int64),
     ]
 
     def as_dict(self):

@@ -251,7 +251,16 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
     }
     case GZ_RUNG_MFMA: {
       MfmaCfg c;
-      if (!mfma_resolve(types, m, n, k, layoutA, layoutB, variant, num_cus, &c)) {
+      MfmaSplit sp;
+      int m_first = m;
+      if (variant == 0 && k > 0 && mfma_resolve_split(types, m, n, k, layoutA, layoutB, num_cus, &sp)) {
+        c = sp.main;
+        m_first = sp.rows_main;
+        plan->tail_rows = m - sp.rows_main;
+        plan->tail_tile_m = sp.tail.bm;
+        plan->tail_tile_n = sp.tail.bn;
+        plan->tail_grid = (int64_t)ceil_div(m - sp.rows_main, sp.tail.bm) * ceil_div(n, sp.tail.bn);
+      } else if (!mfma_resolve(types, m, n, k, layoutA, layoutB, variant, num_cus, &c)) {
         set_error("mfma rung: unknown variant %d", variant);
         return GZ_ERR_UNSUPPORTED;
       }
@@ -260,7 +269,7 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       plan->wave_m = c.bm / c.waves_m; plan->wave_n = c.bn / c.waves_n;
       plan->threads = c.waves_m * c.waves_n * 64;
       plan->lds_bytes = mfma_lds_bytes(c);
-      plan->grid = (int64_t)ceil_div(m, c.bm) * ceil_div(n, c.bn);
+      plan->grid = (int64_t)ceil_div(m_first, c.bm) * ceil_div(n, c.bn);
       if (plan->lds_bytes > lds_per_cu) {
         set_error("mfma variant %d needs %d bytes of LDS, device has %d", c.id, plan->lds_bytes, lds_per_cu);
         return GZ_ERR_UNSUPPORTED;

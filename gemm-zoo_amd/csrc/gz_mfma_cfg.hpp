@@ -51,32 +51,36 @@ inline bool mfma_whole_tiles(const MfmaCfg& c, int in_size, int M, int N, int K)
   return mfma_shape_class(c, in_size, M, N, K, GZ_ROW_MAJOR, GZ_COL_MAJOR) == MFMA_SHAPE_WHOLE;
 }
 
-// Picks the tile configuration by an estimate of the launch's duration:
-//     rounds of tiles over the compute units  x  tile area  x  penalty of the tile shape  x  penalty of the kernel
-// A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does not
-// fill the device, or that leaves a nearly empty last round (N = 4097: 17 tile columns for one column of data),
-// is better served by smaller tiles.  The penalties are measured on MI355X (fp16 4095x4097x1023: 256x256 255 us,
-// 256x128 174 us, 128x128 156 us; 4096x4352x1024 row/row: 256x256 hand-scheduled 79 us, 128x128 general 103 us;
-// bf16 2048^3 row/col: 128x128 30 us, 256x128 41 us, 256x256 51 us).
+// Picks the tile configuration by an estimate of the launch's duration, in units of one round of 256x256 tiles over
+// the compute units (about 105 us at K = 4096 for bf16 on MI355X):
+//     256x256   rounds                      one work-group per compute unit
+//     256x128   0.75 rounds                 one work-group per compute unit, more operand bytes per flop
+//     128x128   0.40 + 0.27 rounds          two work-groups share a compute unit; a lone one cannot fill it
+// (rounds = tiles of that size / compute units, rounded up), times 2.2 where the problem cannot use a direct-to-LDS
+// kernel, times 1.3 / 1.15 for the two smaller tiles on a row-major B (6144 x 6144 x 4096 row/row: 360 / 444 / 319).  A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does
+// not fill the device, or that leaves a nearly empty last round (N = 4097: 17 tile columns for one column of data),
+// is better served by smaller tiles.  Fitted to bf16 row/col squares, K = M = N (us, variants 3 / 4 / 6 =
+// 128x128 / 256x128 / 256x256):
+//     2048: 32 / 41 / 54     2560: 49 / 49 / 65     2816: 57 / 54 / 69     3072: 85 / 106 / 75
+//     3328: 92 / 112 / 82    3584: 117 / 119 / 96   3840: 131 / 130 / 110  6144 (K 4096): 312 / 332 / 318
+// and fp16 4095 x 4097 x 1023 on the predicated kernel: 112 / 143 / 153.
 //   bf16 4096^3 (interleaved runs, us)  v1 117  v2 109  v5 108  v6 109  v7 106
 //   bf16 8192^3                         v1 904  v2 865  v6 845  v7 885
 //   int8 8192^3                         v1 543  v2 558  v5 579  v6 536  v7 582
 // Direct-to-LDS kernels exist for row-major A with whole tiles: hand-scheduled for 256x256 (column-major B: both
 // wave shapes; row-major B: four waves), compiler-scheduled for the smaller tiles; on any other problem the same
 // tile runs the general kernel, so choosing them is always safe.
-inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layoutB, int variant, int num_cus,
-                         MfmaCfg* out) {
-  if (variant < 0 || variant > kNumMfmaCfgs) return false;
-  if (variant > 0) {
-    *out = kMfmaCfgs[variant - 1];
-    return true;
-  }
+inline int mfma_in_size(int types) {
+  return (types == GZ_S8S8S32 || types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) ? 1 : types == GZ_F32F32F32 ? 4 : 2;
+}
+
+// The launcher's own choice for one launch over the whole problem; returns the estimate it was chosen by.
+inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaCfg* out) {
   if (num_cus <= 0) num_cus = 256;
-  const int in_size = (types == GZ_S8S8S32 || types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) ? 1 : types == GZ_F32F32F32 ? 4 : 2;
+  const int in_size = mfma_in_size(types);
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
   // candidates: 256x256 (id 6), 256x128 (id 4), 128x128 (id 3)
   const int cand[3] = {5, 3, 2};
-  const double shape_pen[3] = {1.0, 1.1, 1.25};
   double best = 0;
   int pick = 5;
   for (int i = 0; i < 3; i++) {
@@ -87,7 +91,10 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
     const bool direct = a_rows && types != GZ_F32F32F32 &&
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
-    const double cost = (double)rounds * c.bm * c.bn * shape_pen[i] * (direct ? 1.0 : 2.2);
+    const double shape_cost = i == 0 ? (double)rounds : i == 1 ? 0.75 * rounds : 0.40 + 0.27 * rounds;
+    // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
+    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.3 : 1.15) : 1.0;
+    const double cost = shape_cost * rowb * (direct ? 1.0 : 2.2);
     if (i == 0 || cost < best) {
       best = cost;
       pick = cand[i];
@@ -98,6 +105,54 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
     if (tiles <= 2LL * num_cus) *out = kMfmaCfgs[6];
   }
+  return best;
+}
+
+inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layoutB, int variant, int num_cus,
+                         MfmaCfg* out) {
+  if (variant < 0 || variant > kNumMfmaCfgs) return false;
+  if (variant > 0) {
+    *out = kMfmaCfgs[variant - 1];
+    return true;
+  }
+  (void)mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, out);
+  return true;
+}
+
+// Ragged last round.  When the 256x256 tiles of a problem fill some rounds of the compute units and then leave a
+// last round mostly empty (6144 x 6144: 576 tiles = 2.25 rounds of 256), one launch pays for a whole round more.
+// With a row-major A the rows of the problem can be cut in two launches instead, since row ranges of A, C and D
+// are packed matrices themselves: the first covers as many tile rows as fit whole rounds, with 256x256 tiles, the
+// second the remaining rows with whatever tile the estimate above prefers for them (usually 128x128, which spreads
+// the leftover over all compute units).  Taken when the summed estimate is at least 3 % below the single launch.
+struct MfmaSplit {
+  int rows_main;      // rows of the first launch (a multiple of 256), 0 = no split
+  MfmaCfg main, tail;
+};
+inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaSplit* out) {
+  out->rows_main = 0;
+  if (num_cus <= 0) num_cus = 256;
+  if (layoutA != GZ_ROW_MAJOR || M < 512 || N <= 0 || K <= 0) return false;
+  MfmaCfg single;
+  const double cost_single = mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, &single);
+  const long long tiles_n = (N + 255) / 256, tiles_m = (M + 255) / 256;
+  const long long full = tiles_m * tiles_n / num_cus * num_cus;   // tiles in whole rounds
+  if (full == 0 || full == tiles_m * tiles_n) return false;
+  const long long tile_rows = full / tiles_n;                     // tile rows that fit them
+  if (tile_rows <= 0 || tile_rows * 256 >= M) return false;
+  const int rows_main = (int)(tile_rows * 256);
+  MfmaCfg main_cfg, tail_cfg;
+  double cost_main = mfma_choose(types, rows_main, N, K, layoutA, layoutB, num_cus, &main_cfg);
+  if (main_cfg.bm != 256 || main_cfg.bn != 256) return false;
+  // only where the first launch runs a direct-to-LDS kernel, whose speed the estimate knows well
+  if (types == GZ_F32F32F32 ||
+      mfma_shape_class(main_cfg, mfma_in_size(types), rows_main, N, K, layoutA, layoutB) == MFMA_SHAPE_GENERAL)
+    return false;
+  const double cost_tail = mfma_choose(types, M - rows_main, N, K, layoutA, layoutB, num_cus, &tail_cfg);
+  if (cost_main + cost_tail > 0.97 * cost_single) return false;
+  out->rows_main = rows_main;
+  out->main = main_cfg;
+  out->tail = tail_cfg;
   return true;
 }
 

@@ -1128,13 +1128,8 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   return GZ_OK;
 }
 
-template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
+template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& cfg, hipStream_t s) {
   using in_t = typename Traits<TYPES>::in_t;
-  MfmaCfg cfg;
-  if (!mfma_resolve(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, 256, &cfg)) {
-    set_error("mfma rung: unknown variant %d", variant);
-    return GZ_ERR_UNSUPPORTED;
-  }
   const int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
   switch (cfg.id) {
     case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
@@ -1148,6 +1143,30 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipS
   }
   set_error("mfma rung: variant %d not built", cfg.id);
   return GZ_ERR_UNSUPPORTED;
+}
+
+template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
+  if (variant == 0 && g.K > 0) {
+    // a mostly empty last round of 256x256 tiles: the rows that fill whole rounds first, the rest in a second launch
+    MfmaSplit sp;
+    if (mfma_resolve_split(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, 256, &sp)) {
+      GemmArgs<TYPES> top = g, bottom = g;
+      top.M = sp.rows_main;
+      bottom.M = g.M - sp.rows_main;
+      bottom.A = g.A + (size_t)sp.rows_main * g.K;   // row-major A: a row range is a packed matrix
+      if (g.C) bottom.C = g.C + (size_t)sp.rows_main * g.N;
+      bottom.D = g.D + (size_t)sp.rows_main * g.N;
+      const int st = launch_one<TYPES>(top, sp.main, s);
+      if (st != GZ_OK) return st;
+      return launch_one<TYPES>(bottom, sp.tail, s);
+    }
+  }
+  MfmaCfg cfg;
+  if (!mfma_resolve(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, 256, &cfg)) {
+    set_error("mfma rung: unknown variant %d", variant);
+    return GZ_ERR_UNSUPPORTED;
+  }
+  return launch_one<TYPES>(g, cfg, s);
 }
 
 }  // namespace gz

@@ -103,6 +103,12 @@ typedef struct gz_plan_t {
   int64_t grid;                /* number of work-groups                        */
   int32_t split_k;             /* >1: partial sums reduced in a second pass    */
   int32_t vector_bytes_a, vector_bytes_b; /* widest aligned global access used */
+  /* MFMA rung, launcher's choice only: when the tiles would leave a mostly empty last round of the compute
+   * units, the last tail_rows rows of the problem run in a second launch with their own tile (0: one launch).
+   * rung, tile_*, grid above then describe the first launch (M - tail_rows rows).                          */
+  int32_t tail_rows;
+  int32_t tail_tile_m, tail_tile_n;
+  int64_t tail_grid;
 } gz_plan_t;
 
 /* variant: 0 = launcher's choice; other values select a tile configuration of the rung

@@ -176,3 +176,33 @@ def test_ragged_m_n_on_the_hand_scheduled_kernels(G, types, shape, lb):
     for r in (255, 1024, m - 1):
         ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=(r, r + 1))
         assert np.array_equal(got[r], ref[r])
+
+
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.F16F16F16, O.E4M3E4M3F16])
+@pytest.mark.parametrize("shape,lb", [((4608, 4608, 256), O.COL), ((7168, 7168, 128), O.ROW), ((7168, 7168, 128), O.COL),
+                                      ((4352, 4096, 256), O.ROW)])
+def test_mostly_empty_last_round_runs_as_two_launches(G, types, shape, lb):
+    """324 (or 784) tiles of 256x256 on 256 compute units leave a last round that is mostly empty: the launcher
+    cuts the rows in two launches (whole rounds of 256x256 tiles, then the remaining rows with a smaller tile).
+    The seam between the two row ranges, the first and the last rows are compared with the oracle."""
+    m, n, k = shape
+    p = G.capi.plan(types, m, n, k, O.ROW, lb)
+    assert p.rung == 4 and (p.tile_m, p.tile_n) == (256, 256) and 0 < p.tail_rows < m and p.tail_tile_m in (128, 256)
+    assert (m - p.tail_rows) % 256 == 0 and p.grid == (m - p.tail_rows) // 256 * -(-n // 256) and p.tail_grid > 0
+    # an explicit variant is one launch
+    assert G.capi.plan(types, m, n, k, O.ROW, lb, 4, 6).tail_rows == 0
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+    a, b, ha, hb = device_inputs(G, types, m, n, k, kind, 51)
+    hc = O.fill(m * n, O.OUT_DT[types], kind, 1.0, 53)
+    got = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, -1)
+    seam = m - p.tail_rows
+    for rows in ((0, 8), (seam - 16, seam + 16), (m - 24, m)):
+        ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=rows)
+        assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, shape, lb, rows)
+    # the whole result against the single launch of the same tile (on-device compare would need both; host is enough)
+    one = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, 6)
+    assert np.array_equal(got, one)
+    # beta = 0 with no C
+    got0 = G.run_gemm(types, ha, hb, None, m, n, k, O.ROW, lb, 1, 0, -1)
+    ref = O.gemm(types, ha, hb, None, m, n, k, O.ROW, lb, 1, 0, rows=(seam - 4, seam + 4))
+    assert np.array_equal(got0[seam - 4:seam + 4], ref[seam - 4:seam + 4])
