@@ -57,7 +57,7 @@ inline bool mfma_whole_tiles(const MfmaCfg& c, int in_size, int M, int N, int K)
 //     256x128   0.75 rounds                 one work-group per compute unit, more operand bytes per flop
 //     128x128   0.40 + 0.27 rounds          two work-groups share a compute unit; a lone one cannot fill it
 // (rounds = tiles of that size / compute units, rounded up), times 2.2 where the problem cannot use a direct-to-LDS
-// kernel, times 1.3 / 1.15 for the two smaller tiles on a row-major B (6144 x 6144 x 4096 row/row: 360 / 444 / 319).  A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does
+// kernel, times 1.12 / 1.15 for the two smaller tiles on a row-major B (4096^3 row/row: 152 / 150 / 119).  A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does
 // not fill the device, or that leaves a nearly empty last round (N = 4097: 17 tile columns for one column of data),
 // is better served by smaller tiles.  Fitted to bf16 row/col squares, K = M = N (us, variants 3 / 4 / 6 =
 // 128x128 / 256x128 / 256x256):
@@ -67,9 +67,11 @@ inline bool mfma_whole_tiles(const MfmaCfg& c, int in_size, int M, int N, int K)
 //   bf16 4096^3 (interleaved runs, us)  v1 117  v2 109  v5 108  v6 109  v7 106
 //   bf16 8192^3                         v1 904  v2 865  v6 845  v7 885
 //   int8 8192^3                         v1 543  v2 558  v5 579  v6 536  v7 582
-// Direct-to-LDS kernels exist for row-major A with whole tiles: hand-scheduled for 256x256 (column-major B: both
-// wave shapes; row-major B: four waves), compiler-scheduled for the smaller tiles; on any other problem the same
-// tile runs the general kernel, so choosing them is always safe.
+// "Direct" here means: row-major A and whole tiles (or ragged M / N on 256x256), i.e. no predicated loads and no
+// transposing stores.  256x256 then runs the hand-scheduled direct-to-LDS kernels (column-major B: both wave shapes;
+// row-major B: four waves), the smaller tiles the register-staged kernel without predication (128x128 with a
+// row-major B: a compiler-scheduled direct-to-LDS kernel with transposing LDS reads); on any other problem the same
+// tile runs the predicated kernel, so choosing them is always safe.
 inline int mfma_in_size(int types) {
   return (types == GZ_S8S8S32 || types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) ? 1 : types == GZ_F32F32F32 ? 4 : 2;
 }
@@ -93,7 +95,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     const double shape_cost = i == 0 ? (double)rounds : i == 1 ? 0.75 * rounds : 0.40 + 0.27 * rounds;
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
-    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.3 : 1.15) : 1.0;
+    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : 1.15) : 1.0;
     const double cost = shape_cost * rowb * (direct ? 1.0 : 2.2);
     if (i == 0 || cost < best) {
       best = cost;

@@ -1082,15 +1082,22 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
         return GZ_OK;
       }
     }
-    auto kern = mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
-    GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)dlds));
-    hipLaunchKernelGGL(kern, grid, block, dlds, s, g, tiles_m, tiles_n);
-    GZ_HIP_TRY(hipGetLastError());
-    return GZ_OK;
+    // The compiler-scheduled direct-to-LDS kernel is kept for the eight-wave 256x256 tile only: with four waves the
+    // register-staged kernel below, whose loads and LDS stores are spread between the MFMAs, measured faster on
+    // every tile (interleaved runs, us, direct / register-staged: bf16 2048^3 128x128 28.6 / 27.1, 256x128 39.2 /
+    // 37.0; 4096^3 256x256 130.1 / 121.9; int8 8192^3 512 / 495; fp8 8192^3 479 / 424).
+    if constexpr (WAVES_M * WAVES_N == 8) {
+      auto kern = mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
+      GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)dlds));
+      hipLaunchKernelGGL(kern, grid, block, dlds, s, g, tiles_m, tiles_n);
+      GZ_HIP_TRY(hipGetLastError());
+      return GZ_OK;
+    }
   }
   if (!edge && akc && !bkc) {  // whole tiles, row-major A and B: direct-to-LDS copies, transposing LDS reads for B
-    if constexpr (BN == 128) {
+    // (128x128 only: on 256x128 the register-staged kernel is faster, 2048^3 50.0 / 43.0 us, 4096^3 185 / 150)
+    if constexpr (BM == 128 && BN == 128) {
       const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
       auto kern = mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;
       GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

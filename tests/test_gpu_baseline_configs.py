@@ -130,7 +130,8 @@ def test_c5_skinny_bf16(G, m):
                                         ((512, 384, 256), (128, 128)), ((256, 128, 128), (128, 128))])
 def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile):
     """Row-major A and B (every driver of the reference).  The first shape gives each compute unit a whole 256x256
-    tile (hand-scheduled kernel, transposing LDS reads for B), the others take the 128-wide direct-to-LDS kernels."""
+    tile (hand-scheduled kernel, transposing LDS reads for B), the others take the smaller tiles without predication
+    (256x128: register-staged kernel; 128x128: direct-to-LDS kernel with transposing LDS reads)."""
     m, n, k = shape
     p = G.capi.plan(types, m, n, k, O.ROW, O.ROW)
     assert p.rung == 4 and m % p.tile_m == 0 and n % p.tile_n == 0          # whole tiles: no predicated kernel
