@@ -42,6 +42,8 @@ enum { MFMA_SHAPE_WHOLE = 0, MFMA_SHAPE_RAGGED_MN = 1, MFMA_SHAPE_GENERAL = 2 };
 inline int mfma_shape_class(const MfmaCfg& c, int in_size, int M, int N, int K, int layoutA, int layoutB) {
   const int bk = MFMA_SLAB_BYTES / in_size, epv = 16 / in_size;
   if (K <= 0 || K % bk) return MFMA_SHAPE_GENERAL;
+  // the direct-to-LDS kernels address a tile's rows with 32-bit byte offsets from the tile's first row
+  if ((long long)K * in_size * 256 >= (1LL << 32) || (long long)N * in_size * 256 >= (1LL << 32)) return MFMA_SHAPE_GENERAL;
   if (M % c.bm == 0 && N % c.bn == 0) return MFMA_SHAPE_WHOLE;
   if (layoutA != GZ_ROW_MAJOR) return MFMA_SHAPE_GENERAL;
   if (layoutB == GZ_ROW_MAJOR && N % epv) return MFMA_SHAPE_GENERAL;

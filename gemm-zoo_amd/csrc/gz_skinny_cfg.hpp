@@ -44,6 +44,7 @@ inline bool skinny_supported(int types, int M, int N, int K, int layoutA, int la
   if (types != GZ_BF16BF16F32 && types != GZ_BF16BF16BF16 && types != GZ_F16F16F16) return false;
   if (layoutA != GZ_ROW_MAJOR || layoutB != GZ_COL_MAJOR) return false;
   if (M < 1 || M > SKINNY_MAX_M || N < 1 || K < SKINNY_K_STEP) return false;
+  if ((long long)K * 2 * SKINNY_MAX_M >= (1LL << 32)) return false;  // rows are addressed with 32-bit byte offsets
   return K % SKINNY_K_STEP == 0;
 }
 

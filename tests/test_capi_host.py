@@ -118,8 +118,20 @@ def test_plan_headline_configs(capi):
     assert e.value.status == capi.ERR_UNSUPPORTED
 
 
+def test_plan_split_launch_and_offset_limits(capi):
+    # 324 tiles of 256x256 on 256 compute units: whole rounds first, the remaining rows as a second launch
+    p = capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 0, 1)
+    assert (p.tile_m, p.tile_n, p.grid) == (256, 256, 252) and p.tail_rows == 1024 and p.tail_grid > 0
+    assert capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 1, 1).tail_rows == 0      # column-major A: rows are not packed
+    assert capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 0, 1, capi.RUNG_MFMA, 6).tail_rows == 0
+    assert capi.plan(capi.BF16BF16F32, 4096, 4096, 4096, 0, 1).tail_rows == 0      # exactly one round
+    # the streaming kernels address rows with 32-bit byte offsets: a K of 20 million goes to the tiled rung
+    assert capi.plan(capi.BF16BF16BF16, 64, 64, 20_000_000, 0, 1).rung == capi.RUNG_MFMA
+    assert capi.plan(capi.BF16BF16BF16, 64, 64, 8_000_000, 0, 1).rung == capi.RUNG_SKINNY
+
+
 def test_plan_every_rung_and_type(capi):
-    for types in range(4):
+    for types in range(capi.NUM_TYPES):
         for rung in range(5):
             p = capi.plan(types, 300, 500, 700, 0, 0, rung)
             assert p.rung == rung and p.grid >= 1 and p.threads in (128, 256, 512, 1024)
