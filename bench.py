@@ -24,7 +24,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
-PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "fp8": 5000.0}  # dense MFMA, MI355X
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "fp8": 5000.0, "f32": 157.3}  # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 INFINITY_CACHE_BYTES = 256 * 1000 * 1000
 
@@ -60,13 +60,17 @@ def main() -> int:
     sptr = stream.cuda_stream
 
     IN_T = {capi.S8S8S32: torch.int8, capi.BF16BF16F32: torch.bfloat16, capi.BF16BF16BF16: torch.bfloat16,
-            capi.F16F16F16: torch.float16, capi.E4M3E4M3F16: torch.float8_e4m3fn, capi.E5M2E5M2F16: torch.float8_e5m2}
+            capi.F16F16F16: torch.float16, capi.E4M3E4M3F16: torch.float8_e4m3fn, capi.E5M2E5M2F16: torch.float8_e5m2,
+            capi.F32F32F32: torch.float32}
     OUT_T = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
-             capi.F16F16F16: torch.float16, capi.E4M3E4M3F16: torch.float16, capi.E5M2E5M2F16: torch.float16}
+             capi.F16F16F16: torch.float16, capi.E4M3E4M3F16: torch.float16, capi.E5M2E5M2F16: torch.float16,
+             capi.F32F32F32: torch.float32}
     OUT_DT = {capi.S8S8S32: capi.DT_INT32, capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16,
-              capi.F16F16F16: capi.DT_F16, capi.E4M3E4M3F16: capi.DT_F16, capi.E5M2E5M2F16: capi.DT_F16}
+              capi.F16F16F16: capi.DT_F16, capi.E4M3E4M3F16: capi.DT_F16, capi.E5M2E5M2F16: capi.DT_F16,
+              capi.F32F32F32: capi.DT_F32}
     IN_DT = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
-             capi.F16F16F16: capi.DT_F16, capi.E4M3E4M3F16: capi.DT_E4M3, capi.E5M2E5M2F16: capi.DT_E5M2}
+             capi.F16F16F16: capi.DT_F16, capi.E4M3E4M3F16: capi.DT_E4M3, capi.E5M2E5M2F16: capi.DT_E5M2,
+             capi.F32F32F32: capi.DT_F32}
 
     def make_sets(types, m, n, k, scale_b=1.0, seed0=2025):
         """P rotating (A, B) sets + one D, filled on the device (seeds 2025, 2026, ... as the reference harness)."""
@@ -114,7 +118,7 @@ def main() -> int:
                 # sanity bound only (parity proper lives in tests/): fp32 accumulation in a different order, so allow
                 # 1e-3 of the output scale for fp32 out and one 16-bit ulp at 4 sigma for 16-bit out
                 scale = float(torch.sqrt(torch.tensor(float(k)))) * scale_b
-                tol = (1e-3 if types == capi.BF16BF16F32 else 4e-2) * scale
+                tol = (1e-3 if types in (capi.BF16BF16F32, capi.F32F32F32) else 4e-2) * scale
                 ndiff = capi.compare(d, ref, m * n, dt, tol, sptr)
             if ndiff:
                 raise RuntimeError(f"verification failed: {ndiff} elements differ ({capi.TYPES_NAMES[types]} {m}x{n}x{k})")
@@ -200,13 +204,19 @@ def main() -> int:
         tf8 = 2.0 * m8 ** 3 / (rf["kernel_ms_mean"] * 1e-3) / 1e12
         extras["e4m3_8192_row_row"] = {"tflops": round(tf8, 2), "frac_of_fp8_peak": round(tf8 / PEAK_TFLOPS["fp8"], 4),
                                        "kernel_ms_mean": round(rf["kernel_ms_mean"], 5)}
+        # the type of the reference's own ladder drivers: fp32 4096^3, row-major A and B, full-precision MFMA
+        r32 = timed(capi.F32F32F32, M, N, K, capi.ROW_MAJOR, capi.ROW_MAJOR, 20, 20)
+        t32 = flops / (r32["kernel_ms_mean"] * 1e-3) / 1e12
+        extras["f32_4096_row_row"] = {"tflops": round(t32, 2), "frac_of_f32_peak": round(t32 / PEAK_TFLOPS["f32"], 4),
+                                      "kernel_ms_mean": round(r32["kernel_ms_mean"], 5)}
         # the vendor library beside it (the reference reports cuBLASLt): same operands, same timing, checked the same way
         try:
             functors = importlib.import_module("gemm-zoo_amd.functors")
             for name, (ty, sz, st, wu, lb, sb) in {
                     "hipblaslt_bf16_4096": (capi.BF16BF16F32, 4096, args.steps, args.warmup, capi.COL_MAJOR, 1.0),
                     "hipblaslt_s8_8192": (capi.S8S8S32, 8192, 30, 40, capi.COL_MAJOR, 1.0),
-                    "hipblaslt_e4m3_8192_row_row": (capi.E4M3E4M3F16, 8192, 30, 40, capi.ROW_MAJOR, 0.25)}.items():
+                    "hipblaslt_e4m3_8192_row_row": (capi.E4M3E4M3F16, 8192, 30, 40, capi.ROW_MAJOR, 0.25),
+                    "hipblaslt_f32_4096_row_row": (capi.F32F32F32, 4096, 20, 20, capi.ROW_MAJOR, 1.0)}.items():
                 lt = functors.HipblasLtGemm(ty, sz, sz, sz, capi.ROW_MAJOR, lb)
                 rl = timed(ty, sz, sz, sz, capi.ROW_MAJOR, lb, st, wu, vendor=lt, scale_b=sb)
                 extras[name] = {"tflops": round(2.0 * sz ** 3 / (rl["kernel_ms_mean"] * 1e-3) / 1e12, 2),
