@@ -94,10 +94,10 @@ __host__ __device__ inline float bf16_to_f32(uint16_t h) {
   return __builtin_bit_cast(float, (uint32_t)h << 16);
 }
 __host__ __device__ inline uint16_t f32_to_bf16(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const uint32_t u = __builtin_bit_cast(uint32_t, f);
+  const uint32_t rounded = u + 0x7fffu + ((u >> 16) & 1u);   // round to nearest even
+  const uint32_t quiet = u | 0x00400000u;                    // NaN: keep the sign and payload, set the quiet bit
+  return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded) >> 16);
 }
 __host__ __device__ inline float f16_to_f32(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);

@@ -40,6 +40,14 @@ typedef int i32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F> __device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 template <int TYPES> struct AccVec { using type = f32x16_t; };
 template <> struct AccVec<GZ_S8S8S32> { using type = i32x16_t; };
 
@@ -80,6 +88,62 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, first),
                                                    __builtin_bit_cast(bf16x8_t, second), acc, 0, 0, 0);
   }
+}
+
+// ---------------------------------------------------------------------------
+// Accumulators -> D, shared by every kernel of the rung.  acc[i][j][4 q + e] of a lane is D(m, n + e) with
+//   m = row0 + 32 i + lane % 32,   n = col0 + 32 j + 8 q + 4 (lane / 32)
+// (row0 / col0: first row and column of the wave's sub-tile), so a lane owns four consecutive columns of one
+// row.  Every index into the accumulators is a compile-time constant: written as loops, the larger epilogues
+// (bf16 rounding) were not unrolled and the compiler kept all 256 accumulators in scratch memory, with a store
+// after every MFMA of the main loop.
+//   MODE 0  whole tiles: one 16-byte (fp32 / int32) or 8-byte (16-bit) store per four columns
+//   MODE 1  M or N ragged: rows and columns past the end skipped, element-wise where a row of D is not 16-byte
+//           aligned or ends inside the four columns
+//   MODE 2  element-wise with bounds checks (unaligned D or C)
+// ---------------------------------------------------------------------------
+template <int TYPES, int FM, int FN, int MODE, class Acc>
+__device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc (&acc)[FM][FN], int row0, int col0, int lane) {
+  using out_t = typename Traits<TYPES>::out_t;
+  const int M = g.M, N = g.N;
+  const bool use_c = g.beta != 0;
+  static_for<FM>([&](auto i_c) {
+    constexpr int I = decltype(i_c)::value;
+    const int m = row0 + 32 * I + (lane & 31);
+    static_for<FN>([&](auto j_c) {
+      constexpr int J = decltype(j_c)::value;
+      static_for<4>([&](auto q_c) {
+        constexpr int Q = decltype(q_c)::value;
+        const int n = col0 + 32 * J + 8 * Q + 4 * (lane >> 5);
+        const size_t o = (size_t)m * N + n;
+        const Acc& a = acc[I][J];
+        auto element_wise = [&]() {
+          if (n + 0 < N) g.D[o + 0] = epilogue<TYPES>(a[4 * Q + 0], g.alpha, g.beta, g.C + o + 0);
+          if (n + 1 < N) g.D[o + 1] = epilogue<TYPES>(a[4 * Q + 1], g.alpha, g.beta, g.C + o + 1);
+          if (n + 2 < N) g.D[o + 2] = epilogue<TYPES>(a[4 * Q + 2], g.alpha, g.beta, g.C + o + 2);
+          if (n + 3 < N) g.D[o + 3] = epilogue<TYPES>(a[4 * Q + 3], g.alpha, g.beta, g.C + o + 3);
+        };
+        if constexpr (MODE == 2) {
+          if (m < M) element_wise();
+        } else {
+          if constexpr (MODE == 1) {
+            if (m >= M || n >= N) return;
+            if ((N & 3) != 0 || n + 3 >= N) {
+              element_wise();
+              return;
+            }
+          }
+          out_t cv[4] = {0, 0, 0, 0}, dv[4];
+          if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+          dv[0] = epilogue<TYPES>(a[4 * Q + 0], g.alpha, g.beta, &cv[0]);
+          dv[1] = epilogue<TYPES>(a[4 * Q + 1], g.alpha, g.beta, &cv[1]);
+          dv[2] = epilogue<TYPES>(a[4 * Q + 2], g.alpha, g.beta, &cv[2]);
+          dv[3] = epilogue<TYPES>(a[4 * Q + 3], g.alpha, g.beta, &cv[3]);
+          __builtin_memcpy(g.D + o, dv, sizeof(dv));
+        }
+      });
+    });
+  });
 }
 
 // MFMA instructions behind one mfma32 call
@@ -463,36 +527,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // Epilogue.  acc[i][j][4*q + e] is D(m, n + e) with
-  //   m = m0 + wm*WM + 32 i + lane%32,  n = n0 + wn*WN + 32 j + 8 q + 4 (lane/32).
-  const int N = g.N;
-  const bool use_c = g.beta != 0;
-#pragma unroll
-  for (int i = 0; i < FM; i++) {
-    const int m = m0 + wm * WM + 32 * i + (lane & 31);
-#pragma unroll
-    for (int j = 0; j < FN; j++) {
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
-        const size_t o = (size_t)m * N + n;
-        if constexpr (!EDGE) {
-          out_t cv[4] = {0, 0, 0, 0}, dv[4];
-          if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
-#pragma unroll
-          for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
-          if constexpr (sizeof(out_t) == 4) *reinterpret_cast<u32x4_t*>(g.D + o) = __builtin_bit_cast(u32x4_t, dv);
-          else *reinterpret_cast<u32x2_t*>(g.D + o) = __builtin_bit_cast(u32x2_t, dv);
-        } else {
-          if (m < g.M) {
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              if (n + e < N) g.D[o + e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, g.C + o + e);
-          }
-        }
-      }
-    }
-  }
+  store_accumulators<TYPES, FM, FN, EDGE ? 2 : 0>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -710,25 +745,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // Epilogue: same register layout as the staged kernel.
-  const bool use_c = g.beta != 0;
-#pragma unroll
-  for (int i = 0; i < FM; i++) {
-    const int m = m0 + wm * WM + 32 * i + (lane & 31);
-#pragma unroll
-    for (int j = 0; j < FN; j++) {
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
-        const size_t o = (size_t)m * N + n;
-        out_t cv[4] = {0, 0, 0, 0}, dv[4];
-        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
-#pragma unroll
-        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
-        __builtin_memcpy(g.D + o, dv, sizeof(dv));
-      }
-    }
-  }
+  store_accumulators<TYPES, FM, FN, 0>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -750,14 +767,6 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 // freed by that barrier are issued in step 3 of slab kt and step 0 of slab kt+1, so they have two more
 // steps to land.
 // ---------------------------------------------------------------------------
-template <class F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, class F> __device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 template <int OFF> __device__ __forceinline__ void asm_ds_read16(u32x4_t& dst, uint32_t addr) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
 }
@@ -986,26 +995,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
   });
 
-  // Epilogue: same register layout as the staged kernel.
-  const int N = g.N;
-  const bool use_c = g.beta != 0;
-#pragma unroll
-  for (int i = 0; i < FM; i++) {
-    const int m = m0 + wm * WM + 32 * i + (lane & 31);
-#pragma unroll
-    for (int j = 0; j < FN; j++) {
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
-        const size_t o = (size_t)m * N + n;
-        out_t cv[4] = {0, 0, 0, 0}, dv[4];
-        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
-#pragma unroll
-        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
-        __builtin_memcpy(g.D + o, dv, sizeof(dv));
-      }
-    }
-  }
+  store_accumulators<TYPES, FM, FN, 0>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 }  // namespace gz

@@ -377,34 +377,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
   });
 
-  // Epilogue: same register layout as the staged kernel.
-  const bool use_c = g.beta != 0;
-#pragma unroll
-  for (int i = 0; i < FM; i++) {
-    const int m = m0 + wm * WM + 32 * i + (lane & 31);
-#pragma unroll
-    for (int j = 0; j < FN; j++) {
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int n = n0 + wn * WN + 32 * j + 8 * q + 4 * (lane >> 5);
-        const size_t o = (size_t)m * N + n;
-        if constexpr (RAGGED) {
-          if (m >= M || n >= N) continue;
-          if ((N & 3) != 0 || n + 3 >= N) {  // rows of D not 16-byte aligned, or the row ends inside these four
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              if (n + e < N) g.D[o + e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, g.C + o + e);
-            continue;
-          }
-        }
-        out_t cv[4] = {0, 0, 0, 0}, dv[4];
-        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
-#pragma unroll
-        for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][j][4 * q + e], g.alpha, g.beta, &cv[e]);
-        __builtin_memcpy(g.D + o, dv, sizeof(dv));
-      }
-    }
-  }
+  store_accumulators<TYPES, FM, FN, RAGGED ? 1 : 0>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 }  // namespace gz
