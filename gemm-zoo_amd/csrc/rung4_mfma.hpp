@@ -155,18 +155,21 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
 // region (row pitch COLS * 4 + 16 bytes), reads it back row by row and stores runs of COLS * sizeof(out) contiguous
 // bytes (also the loads of C).  `region` is this wave's 32 x (COLS * 4 + 16) bytes; the caller has made sure that no
 // wave still reads operands from LDS.
-template <int TYPES, int FM, int FN, class Acc>
+template <int TYPES, int FM, int FN, bool RAGGED = false, class Acc>
 __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g, Acc (&acc)[FM][FN], int row0, int col0,
                                                        int lane, char* region) {
   using out_t = typename Traits<TYPES>::out_t;
   using acc_t = typename Traits<TYPES>::acc_t;
   constexpr int COLS = FN * 32, PITCH_E = COLS * 4 + 16;
   constexpr int LPR = COLS / 4, RPI = 64 / LPR, NI = 32 / RPI;   // lanes per row, rows per instruction, instructions
-  const int N = g.N;
+  const int M = g.M, N = g.N;
   const bool use_c = g.beta != 0;
   char* wr = region + (lane & 31) * PITCH_E + (lane >> 5) * 16;
   const char* rd = region + (lane / LPR) * PITCH_E + (lane % LPR) * 16;
   const int n = col0 + (lane % LPR) * 4;
+  // RAGGED: M or N is not a multiple of the tile; rows and columns past the end are skipped, and where a row of D
+  // is not 16-byte aligned or ends inside this lane's four columns they are written one by one
+  const bool vec_ok = !RAGGED || ((N & 3) == 0 && n + 3 < N);
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
     // the block's values of C first: their latency passes while the accumulators go through LDS
@@ -174,7 +177,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
     static_for<NI>([&](auto t_c) {
       constexpr int T = decltype(t_c)::value;
       cv[T][0] = cv[T][1] = cv[T][2] = cv[T][3] = 0;
-      if (use_c) __builtin_memcpy(cv[T], g.C + (size_t)(row0 + 32 * I + T * RPI + lane / LPR) * N + n, sizeof(cv[T]));
+      const int m = row0 + 32 * I + T * RPI + lane / LPR;
+      if (use_c && vec_ok && (!RAGGED || m < M)) __builtin_memcpy(cv[T], g.C + (size_t)m * N + n, sizeof(cv[T]));
     });
     static_for<FN>([&](auto j_c) {
       constexpr int J = decltype(j_c)::value;
@@ -191,7 +195,18 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       constexpr int T = decltype(t_c)::value;
       acc_t v[4];
       __builtin_memcpy(v, rd + T * RPI * PITCH_E, 16);
-      const size_t o = (size_t)(row0 + 32 * I + T * RPI + lane / LPR) * N + n;
+      const int m = row0 + 32 * I + T * RPI + lane / LPR;
+      const size_t o = (size_t)m * N + n;
+      if constexpr (RAGGED) {
+        if (m >= M || n >= N) return;
+        if (!vec_ok) {
+          if (n + 0 < N) g.D[o + 0] = epilogue<TYPES>(v[0], g.alpha, g.beta, g.C + o + 0);
+          if (n + 1 < N) g.D[o + 1] = epilogue<TYPES>(v[1], g.alpha, g.beta, g.C + o + 1);
+          if (n + 2 < N) g.D[o + 2] = epilogue<TYPES>(v[2], g.alpha, g.beta, g.C + o + 2);
+          if (n + 3 < N) g.D[o + 3] = epilogue<TYPES>(v[3], g.alpha, g.beta, g.C + o + 3);
+          return;
+        }
+      }
       out_t dv[4];
       dv[0] = epilogue<TYPES>(v[0], g.alpha, g.beta, &cv[T][0]);
       dv[1] = epilogue<TYPES>(v[1], g.alpha, g.beta, &cv[T][1]);

@@ -377,13 +377,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
   });
 
-  if constexpr (RAGGED) {
-    store_accumulators<TYPES, FM, FN, 1>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
-  } else {
-    static_assert(NW * epilogue_region_bytes<FN>() <= NST * STAGE_BYTES, "the epilogue reuses the operand buffers");
-    __syncthreads();   // no wave reads operands any more and no copy is in flight
-    store_accumulators_lds<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
-  }
+  static_assert(NW * epilogue_region_bytes<FN>() <= NST * STAGE_BYTES, "the epilogue reuses the operand buffers");
+  __syncthreads();   // no wave reads operands any more and no copy is in flight
+  store_accumulators_lds<TYPES, FM, FN, RAGGED>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
 }
 
 }  // namespace gz
