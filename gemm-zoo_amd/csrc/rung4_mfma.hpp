@@ -97,15 +97,12 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
 // row.  Every index into the accumulators is a compile-time constant: written as loops, the larger epilogues
 // (bf16 rounding) were not unrolled and the compiler kept all 256 accumulators in scratch memory, with a store
 // after every MFMA of the main loop.
-//   MODE 0  whole tiles: one 16-byte (fp32 / int32) or 8-byte (16-bit) store per four columns
-//   MODE 1  M or N ragged: rows and columns past the end skipped, element-wise where a row of D is not 16-byte
-//           aligned or ends inside the four columns
-//   MODE 2  element-wise with bounds checks (unaligned D or C)
+// Whole tiles, straight from the registers: one 16-byte (fp32 / int32) or 8-byte (16-bit) store per four columns.
 // ---------------------------------------------------------------------------
-template <int TYPES, int FM, int FN, int MODE, class Acc>
+template <int TYPES, int FM, int FN, class Acc>
 __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc (&acc)[FM][FN], int row0, int col0, int lane) {
   using out_t = typename Traits<TYPES>::out_t;
-  const int M = g.M, N = g.N;
+  const int N = g.N;
   const bool use_c = g.beta != 0;
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
@@ -117,36 +114,19 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
         const int n = col0 + 32 * J + 8 * Q + 4 * (lane >> 5);
         const size_t o = (size_t)m * N + n;
         const Acc& a = acc[I][J];
-        auto element_wise = [&]() {
-          if (n + 0 < N) g.D[o + 0] = epilogue<TYPES>(a[4 * Q + 0], g.alpha, g.beta, g.C + o + 0);
-          if (n + 1 < N) g.D[o + 1] = epilogue<TYPES>(a[4 * Q + 1], g.alpha, g.beta, g.C + o + 1);
-          if (n + 2 < N) g.D[o + 2] = epilogue<TYPES>(a[4 * Q + 2], g.alpha, g.beta, g.C + o + 2);
-          if (n + 3 < N) g.D[o + 3] = epilogue<TYPES>(a[4 * Q + 3], g.alpha, g.beta, g.C + o + 3);
-        };
-        if constexpr (MODE == 2) {
-          if (m < M) element_wise();
-        } else {
-          if constexpr (MODE == 1) {
-            if (m >= M || n >= N) return;
-            if ((N & 3) != 0 || n + 3 >= N) {
-              element_wise();
-              return;
-            }
-          }
-          out_t cv[4] = {0, 0, 0, 0}, dv[4];
-          if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
-          dv[0] = epilogue<TYPES>(a[4 * Q + 0], g.alpha, g.beta, &cv[0]);
-          dv[1] = epilogue<TYPES>(a[4 * Q + 1], g.alpha, g.beta, &cv[1]);
-          dv[2] = epilogue<TYPES>(a[4 * Q + 2], g.alpha, g.beta, &cv[2]);
-          dv[3] = epilogue<TYPES>(a[4 * Q + 3], g.alpha, g.beta, &cv[3]);
-          __builtin_memcpy(g.D + o, dv, sizeof(dv));
-        }
+        out_t cv[4] = {0, 0, 0, 0}, dv[4];
+        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+        dv[0] = epilogue<TYPES>(a[4 * Q + 0], g.alpha, g.beta, &cv[0]);
+        dv[1] = epilogue<TYPES>(a[4 * Q + 1], g.alpha, g.beta, &cv[1]);
+        dv[2] = epilogue<TYPES>(a[4 * Q + 2], g.alpha, g.beta, &cv[2]);
+        dv[3] = epilogue<TYPES>(a[4 * Q + 3], g.alpha, g.beta, &cv[3]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
       });
     });
   });
 }
 
-// Whole tiles: the same through LDS, so that a store instruction writes whole cache lines.  Straight from the
+// The same through LDS, so that a store instruction writes whole cache lines.  Straight from the
 // accumulators a wave's store covers 32 rows x 32 bytes, and the output - 64 MiB for fp32 4096^2, 256 MiB for int32
 // 8192^2, written by all compute units at the same moment - left the device at about 3 TB/s (a launch with K = 64:
 // 20-24 us; int8 8192 x 8192 x 128: 89 us).  Measured in interleaved runs against the direct stores, beta = 0: bf16
@@ -167,9 +147,12 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   char* wr = region + (lane & 31) * PITCH_E + (lane >> 5) * 16;
   const char* rd = region + (lane / LPR) * PITCH_E + (lane % LPR) * 16;
   const int n = col0 + (lane % LPR) * 4;
-  // RAGGED: M or N is not a multiple of the tile; rows and columns past the end are skipped, and where a row of D
-  // is not 16-byte aligned or ends inside this lane's four columns they are written one by one
-  const bool vec_ok = !RAGGED || ((N & 3) == 0 && n + 3 < N);
+  // RAGGED: M or N need not be multiples of the tile and D / C need not be aligned.  Rows and columns past the end
+  // are skipped.  Where the rows of D (and C) are whole, aligned groups of four elements the stores stay vectors;
+  // otherwise the block is written one element per lane with the lanes along a row, which is still whole cache
+  // lines per instruction (fp16 4095 x 4097 x 63 took 65 us with four scattered 2-byte stores per lane).
+  constexpr uintptr_t VEC_ALIGN = 4 * sizeof(out_t) - 1;
+  const bool vec = !RAGGED || ((N & 3) == 0 && ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & VEC_ALIGN) == 0);
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
     // the block's values of C first: their latency passes while the accumulators go through LDS
@@ -178,7 +161,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       constexpr int T = decltype(t_c)::value;
       cv[T][0] = cv[T][1] = cv[T][2] = cv[T][3] = 0;
       const int m = row0 + 32 * I + T * RPI + lane / LPR;
-      if (use_c && vec_ok && (!RAGGED || m < M)) __builtin_memcpy(cv[T], g.C + (size_t)m * N + n, sizeof(cv[T]));
+      if (use_c && vec && (!RAGGED || (m < M && n < N))) __builtin_memcpy(cv[T], g.C + (size_t)m * N + n, sizeof(cv[T]));
     });
     static_for<FN>([&](auto j_c) {
       constexpr int J = decltype(j_c)::value;
@@ -191,29 +174,37 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
     });
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    static_for<NI>([&](auto t_c) {
-      constexpr int T = decltype(t_c)::value;
-      acc_t v[4];
-      __builtin_memcpy(v, rd + T * RPI * PITCH_E, 16);
-      const int m = row0 + 32 * I + T * RPI + lane / LPR;
-      const size_t o = (size_t)m * N + n;
-      if constexpr (RAGGED) {
-        if (m >= M || n >= N) return;
-        if (!vec_ok) {
-          if (n + 0 < N) g.D[o + 0] = epilogue<TYPES>(v[0], g.alpha, g.beta, g.C + o + 0);
-          if (n + 1 < N) g.D[o + 1] = epilogue<TYPES>(v[1], g.alpha, g.beta, g.C + o + 1);
-          if (n + 2 < N) g.D[o + 2] = epilogue<TYPES>(v[2], g.alpha, g.beta, g.C + o + 2);
-          if (n + 3 < N) g.D[o + 3] = epilogue<TYPES>(v[3], g.alpha, g.beta, g.C + o + 3);
-          return;
+    if (vec) {
+      static_for<NI>([&](auto t_c) {
+        constexpr int T = decltype(t_c)::value;
+        acc_t v[4];
+        __builtin_memcpy(v, rd + T * RPI * PITCH_E, 16);
+        const int m = row0 + 32 * I + T * RPI + lane / LPR;
+        const size_t o = (size_t)m * N + n;
+        if constexpr (RAGGED) {
+          if (m >= M || n >= N) return;   // N is a multiple of four here: the lane's four columns end together
+        }
+        out_t dv[4];
+        dv[0] = epilogue<TYPES>(v[0], g.alpha, g.beta, &cv[T][0]);
+        dv[1] = epilogue<TYPES>(v[1], g.alpha, g.beta, &cv[T][1]);
+        dv[2] = epilogue<TYPES>(v[2], g.alpha, g.beta, &cv[T][2]);
+        dv[3] = epilogue<TYPES>(v[3], g.alpha, g.beta, &cv[T][3]);
+        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+      });
+    } else if constexpr (RAGGED) {
+      for (int r = 0; r < 32; r++) {
+        const int m = row0 + 32 * I + r;
+        if (m >= M) break;
+#pragma unroll
+        for (int c0 = 0; c0 < COLS; c0 += 64) {
+          const int nn = col0 + c0 + lane;
+          acc_t v;
+          __builtin_memcpy(&v, region + r * PITCH_E + (c0 + lane) * 4, 4);
+          const size_t o = (size_t)m * N + nn;
+          if (nn < N) g.D[o] = epilogue<TYPES>(v, g.alpha, g.beta, g.C + o);
         }
       }
-      out_t dv[4];
-      dv[0] = epilogue<TYPES>(v[0], g.alpha, g.beta, &cv[T][0]);
-      dv[1] = epilogue<TYPES>(v[1], g.alpha, g.beta, &cv[T][1]);
-      dv[2] = epilogue<TYPES>(v[2], g.alpha, g.beta, &cv[T][2]);
-      dv[3] = epilogue<TYPES>(v[3], g.alpha, g.beta, &cv[T][3]);
-      __builtin_memcpy(g.D + o, dv, sizeof(dv));
-    });
+    }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   });
@@ -601,13 +592,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  if constexpr (EDGE) {
-    store_accumulators<TYPES, FM, FN, 2>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
-  } else {
-    static_assert(NT / 64 * epilogue_region_bytes<FN>() <= 2 * STAGE_BYTES, "the epilogue reuses the operand buffers");
-    __syncthreads();   // every wave has its last fragments: the operand buffers are free
-    store_accumulators_lds<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
-  }
+  static_assert(NT / 64 * epilogue_region_bytes<FN>() <= 2 * STAGE_BYTES, "the epilogue reuses the operand buffers");
+  __syncthreads();   // every wave has its last fragments: the operand buffers are free
+  store_accumulators_lds<TYPES, FM, FN, EDGE>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
 }
 
 // ---------------------------------------------------------------------------
@@ -825,7 +812,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  store_accumulators<TYPES, FM, FN, 0>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
+  store_accumulators<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -1075,7 +1062,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
   });
 
-  store_accumulators<TYPES, FM, FN, 0>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
+  store_accumulators<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 }  // namespace gz
