@@ -812,7 +812,10 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  store_accumulators<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
+  static_assert(NW * epilogue_region_bytes<FN>() <= 2 * STAGE_BYTES, "the epilogue reuses the operand buffers");
+  __builtin_amdgcn_s_waitcnt(0x0070);  // no copy of this wave is still on its way into LDS
+  __syncthreads();
+  store_accumulators_lds<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
 }
 
 // ---------------------------------------------------------------------------
