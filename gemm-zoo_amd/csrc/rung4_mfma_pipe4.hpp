@@ -331,7 +331,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       static_for<B_PW>([&](auto t) { copy_b(t, 3, m3); });
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");  // simple and safe: the prologue is short
+  // half-slab 0 has landed (what was issued after it may still be on its way: the first barriers of the loop wait
+  // for the following half-slabs in turn)
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(DEEP ? 3 * NCP : 2 * NCP + A_PW) : "memory");
   static_for<NRD>([&](auto r) { read_one(I0{}, r, 0, 0); });
   if constexpr (DEEP) static_for<NRD>([&](auto r) { read_one(I1{}, r, 0, 1); });
 
