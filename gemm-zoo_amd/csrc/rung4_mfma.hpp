@@ -205,8 +205,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         }
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    // no wait here: the LDS executes a wave's instructions in order, so the next block's stores, issued right
+    // behind these loads, cannot overtake them, and they land while this block's values are on their way out
   });
 }
 template <int FN> constexpr int epilogue_region_bytes() { return 32 * (FN * 32 * 4 + 16); }
