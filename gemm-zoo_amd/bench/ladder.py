@@ -23,7 +23,8 @@ sys.path.insert(0, str(ROOT))
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--types", default="bf16bf16f32",
-                    choices=["s8s8s32", "bf16bf16f32", "bf16bf16bf16", "f16f16f16", "f32f32f32", "e4m3e4m3f16", "e5m2e5m2f16"])
+                    choices=["s8s8s32", "bf16bf16f32", "bf16bf16bf16", "f16f16f16", "f32f32f32", "e4m3e4m3f16", "e5m2e5m2f16",
+                             "bf16bf16bf16_acc16", "f16f16f16_acc16"])
     ap.add_argument("--size", type=int, default=4096, help="M = N = K")
     ap.add_argument("--layout-a", default="row", choices=["row", "col"])
     ap.add_argument("--layout-b", default="col", choices=["row", "col"])
@@ -42,14 +43,16 @@ def main() -> int:
     f8 = (capi.E4M3E4M3F16, capi.E5M2E5M2F16)
     tin = {capi.S8S8S32: torch.int8, capi.BF16BF16F32: torch.bfloat16, capi.BF16BF16BF16: torch.bfloat16,
            capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32, capi.E4M3E4M3F16: torch.float8_e4m3fn,
-           capi.E5M2E5M2F16: torch.float8_e5m2}[types]
+           capi.E5M2E5M2F16: torch.float8_e5m2, capi.BF16BF16BF16_ACC16: torch.bfloat16,
+           capi.F16F16F16_ACC16: torch.float16}[types]
     tout = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
-            capi.F32F32F32: torch.float32}.get(types, torch.float16)
+            capi.BF16BF16BF16_ACC16: torch.bfloat16, capi.F32F32F32: torch.float32}.get(types, torch.float16)
     in_dt = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
              capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32, capi.E4M3E4M3F16: capi.DT_E4M3,
-             capi.E5M2E5M2F16: capi.DT_E5M2}[types]
+             capi.E5M2E5M2F16: capi.DT_E5M2, capi.BF16BF16BF16_ACC16: capi.DT_BF16,
+             capi.F16F16F16_ACC16: capi.DT_F16}[types]
     out_dt = {capi.S8S8S32: capi.DT_INT32, capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16,
-              capi.F32F32F32: capi.DT_F32}.get(types, capi.DT_F16)
+              capi.BF16BF16BF16_ACC16: capi.DT_BF16, capi.F32F32F32: capi.DT_F32}.get(types, capi.DT_F16)
     la = capi.ROW_MAJOR if args.layout_a == "row" else capi.COL_MAJOR
     lb = capi.ROW_MAJOR if args.layout_b == "row" else capi.COL_MAJOR
     n = args.size

@@ -32,7 +32,7 @@ PRODUCT_SOURCES = [
     "gz_api.hip", "gz_fill_compare.hip", "rung0_naive.hip", "rung1_coalesced.hip",
     "rung23_lds.hip", "rung4_mfma_s8s8s32.hip", "rung4_mfma_bf16bf16f32.hip", "rung4_mfma_bf16bf16bf16.hip",
     "rung4_mfma_f16f16f16.hip", "rung4_mfma_f32f32f32.hip", "rung4_mfma_e4m3e4m3f16.hip",
-    "rung4_mfma_e5m2e5m2f16.hip", "rung5_skinny.hip",
+    "rung4_mfma_e5m2e5m2f16.hip", "rung4_mfma_acc16.hip", "rung5_skinny.hip",
 ]
 COMPARATOR_SOURCES = ["gz_hipblaslt.cpp"]
 

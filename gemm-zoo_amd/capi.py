@@ -15,20 +15,24 @@ LIB_PATH = _HERE / "lib" / "libgemmzoo.so"
 OK, ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_MISMATCH = 0, 1, 2, 3, 4
 ROW_MAJOR, COL_MAJOR = 0, 1
 S8S8S32, BF16BF16F32, BF16BF16BF16, F16F16F16, F32F32F32, E4M3E4M3F16, E5M2E5M2F16 = 0, 1, 2, 3, 4, 5, 6
-NUM_TYPES = 7
+BF16BF16BF16_ACC16, F16F16F16_ACC16 = 7, 8   # opt-in: the reference kernels' 16-bit running sums
+NUM_TYPES = 9
 RUNG_AUTO, RUNG_NAIVE, RUNG_COALESCED, RUNG_LDS_TILED, RUNG_DOUBLE_BUFFERED, RUNG_MFMA, RUNG_SKINNY = -1, 0, 1, 2, 3, 4, 5
 NUM_RUNGS = 6
 DT_INT8, DT_BF16, DT_F16, DT_F32, DT_INT32, DT_E4M3, DT_E5M2 = 0, 1, 2, 3, 4, 5, 6
 FILL_INT8_UNIFORM, FILL_NORMAL, FILL_UNIFORM_PM1, FILL_SMALL_INT = 0, 1, 2, 3
 
 TYPES_NAMES = {S8S8S32: "s8s8s32", BF16BF16F32: "bf16bf16f32", BF16BF16BF16: "bf16bf16bf16", F16F16F16: "f16f16f16",
-               F32F32F32: "f32f32f32", E4M3E4M3F16: "e4m3e4m3f16", E5M2E5M2F16: "e5m2e5m2f16"}
-IN_SIZE = {S8S8S32: 1, BF16BF16F32: 2, BF16BF16BF16: 2, F16F16F16: 2, F32F32F32: 4, E4M3E4M3F16: 1, E5M2E5M2F16: 1}
-OUT_SIZE = {S8S8S32: 4, BF16BF16F32: 4, BF16BF16BF16: 2, F16F16F16: 2, F32F32F32: 4, E4M3E4M3F16: 2, E5M2E5M2F16: 2}
+               F32F32F32: "f32f32f32", E4M3E4M3F16: "e4m3e4m3f16", E5M2E5M2F16: "e5m2e5m2f16",
+               BF16BF16BF16_ACC16: "bf16bf16bf16_acc16", F16F16F16_ACC16: "f16f16f16_acc16"}
+IN_SIZE = {S8S8S32: 1, BF16BF16F32: 2, BF16BF16BF16: 2, F16F16F16: 2, F32F32F32: 4, E4M3E4M3F16: 1, E5M2E5M2F16: 1,
+           BF16BF16BF16_ACC16: 2, F16F16F16_ACC16: 2}
+OUT_SIZE = {S8S8S32: 4, BF16BF16F32: 4, BF16BF16BF16: 2, F16F16F16: 2, F32F32F32: 4, E4M3E4M3F16: 2, E5M2E5M2F16: 2,
+            BF16BF16BF16_ACC16: 2, F16F16F16_ACC16: 2}
 
 EXPORTS = [
     "gz_gemm_s8s8s32", "gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16", "gz_gemm_f32f32f32",
-    "gz_gemm_e4m3e4m3f16", "gz_gemm_e5m2e5m2f16", "gz_gemm",
+    "gz_gemm_e4m3e4m3f16", "gz_gemm_e5m2e5m2f16", "gz_gemm_bf16bf16bf16_acc16", "gz_gemm_f16f16f16_acc16", "gz_gemm",
     "gz_plan", "gz_variant_count", "gz_rung_name", "gz_types_name", "gz_fill", "gz_compare", "gz_compare_rel",
     "gz_last_error", "gz_version",
 ]
@@ -67,7 +71,8 @@ def _load():
     common = [vp, vp, vp, vp, i64, i64, i64, i32, i32]
     lib.gz_gemm_s8s8s32.argtypes = common + [C.c_int32, C.c_int32, i32, i32, vp]
     for name in ("gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16", "gz_gemm_f32f32f32",
-                 "gz_gemm_e4m3e4m3f16", "gz_gemm_e5m2e5m2f16"):
+                 "gz_gemm_e4m3e4m3f16", "gz_gemm_e5m2e5m2f16", "gz_gemm_bf16bf16bf16_acc16",
+                 "gz_gemm_f16f16f16_acc16"):
         getattr(lib, name).argtypes = common + [f32, f32, i32, i32, vp]
     lib.gz_gemm.argtypes = [i32] + common + [f64, f64, i32, i32, vp]
     lib.gz_plan.argtypes = [i32, i64, i64, i64, i32, i32, i32, i32, i32, i32, C.POINTER(Plan)]
@@ -114,7 +119,8 @@ def gemm(types: int, a, b, c, d, m: int, n: int, k: int, layout_a: int = ROW_MAJ
     fn = {S8S8S32: lib.gz_gemm_s8s8s32, BF16BF16F32: lib.gz_gemm_bf16bf16f32,
           BF16BF16BF16: lib.gz_gemm_bf16bf16bf16, F16F16F16: lib.gz_gemm_f16f16f16,
           F32F32F32: lib.gz_gemm_f32f32f32, E4M3E4M3F16: lib.gz_gemm_e4m3e4m3f16,
-          E5M2E5M2F16: lib.gz_gemm_e5m2e5m2f16}.get(types)
+          E5M2E5M2F16: lib.gz_gemm_e5m2e5m2f16, BF16BF16BF16_ACC16: lib.gz_gemm_bf16bf16bf16_acc16,
+          F16F16F16_ACC16: lib.gz_gemm_f16f16f16_acc16}.get(types)
     if fn is None:
         raise GzError(ERR_BAD_ARG, f"unknown type bundle {types}")
     if types == S8S8S32:

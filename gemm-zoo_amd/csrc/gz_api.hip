@@ -27,7 +27,8 @@ int hip_fail(hipError_t e, const char* what) {
 
 static const char* kRungNames[GZ_NUM_RUNGS] = {"naive", "coalesced", "lds_tiled", "double_buffered", "mfma", "skinny"};
 static const char* kTypesNames[GZ_NUM_TYPES] = {"s8s8s32",   "bf16bf16f32", "bf16bf16bf16", "f16f16f16",
-                                                "f32f32f32", "e4m3e4m3f16", "e5m2e5m2f16"};
+                                                "f32f32f32", "e4m3e4m3f16", "e5m2e5m2f16",
+                                                "bf16bf16bf16_acc16", "f16f16f16_acc16"};
 
 static int in_size(int types) { return (types == GZ_S8S8S32 || is_fp8(types)) ? 1 : types == GZ_F32F32F32 ? 4 : 2; }
 static int out_size(int types) {
@@ -160,6 +161,20 @@ int gz_gemm_e5m2e5m2f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, u
                              round_out<GZ_E5M2E5M2F16>(beta), rung, variant, stream);
 }
 
+int gz_gemm_bf16bf16bf16_acc16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int64_t M,
+                               int64_t N, int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung,
+                               int variant, gz_stream stream) {
+  return run<GZ_BF16BF16BF16_ACC16>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<GZ_BF16BF16BF16_ACC16>(alpha),
+                                    round_out<GZ_BF16BF16BF16_ACC16>(beta), rung, variant, stream);
+}
+
+int gz_gemm_f16f16f16_acc16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int64_t M,
+                            int64_t N, int64_t K, int layoutA, int layoutB, float alpha, float beta, int rung,
+                            int variant, gz_stream stream) {
+  return run<GZ_F16F16F16_ACC16>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<GZ_F16F16F16_ACC16>(alpha),
+                                 round_out<GZ_F16F16F16_ACC16>(beta), rung, variant, stream);
+}
+
 int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K,
             int layoutA, int layoutB, double alpha, double beta, int rung, int variant, gz_stream stream) {
   switch (types) {
@@ -189,6 +204,12 @@ int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int
     case GZ_E5M2E5M2F16:
       return gz_gemm_e5m2e5m2f16((const uint8_t*)A, (const uint8_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
                                  layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
+    case GZ_BF16BF16BF16_ACC16:
+      return gz_gemm_bf16bf16bf16_acc16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N,
+                                        K, layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
+    case GZ_F16F16F16_ACC16:
+      return gz_gemm_f16f16f16_acc16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
+                                     layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
     default: break;
   }
   set_error("unknown type bundle %d", types);
@@ -199,8 +220,8 @@ int gz_variant_count(int types, int rung) {
   if (types < 0 || types >= GZ_NUM_TYPES) return 0;
   switch (rung) {
     case GZ_RUNG_NAIVE: case GZ_RUNG_COALESCED: case GZ_RUNG_LDS_TILED: case GZ_RUNG_DOUBLE_BUFFERED: return 1;
-    case GZ_RUNG_MFMA: return kNumMfmaCfgs;
-    case GZ_RUNG_SKINNY: return (types == GZ_S8S8S32 || types == GZ_F32F32F32 || is_fp8(types)) ? 0 : 1;
+    case GZ_RUNG_MFMA: return is_acc16(types) ? 1 : kNumMfmaCfgs;
+    case GZ_RUNG_SKINNY: return (types == GZ_S8S8S32 || types == GZ_F32F32F32 || is_fp8(types) || is_acc16(types)) ? 0 : 1;
     default: return 0;
   }
 }
@@ -250,6 +271,14 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       return GZ_OK;
     }
     case GZ_RUNG_MFMA: {
+      if (is_acc16(types)) {   // one kernel: 128 x 128 tile, four waves of 64 x 64, slabs of 32 k (rung4_mfma_acc16.hip)
+        if (variant > 1) { set_error("mfma rung has a single variant for the 16-bit running-sum modes"); return GZ_ERR_UNSUPPORTED; }
+        plan->variant = 1;
+        plan->tile_m = 128; plan->tile_n = 128; plan->tile_k = 32; plan->wave_m = 64; plan->wave_n = 64;
+        plan->threads = 256; plan->lds_bytes = 256 * (64 + 16);
+        plan->grid = (int64_t)ceil_div(m, 128) * ceil_div(n, 128);
+        return GZ_OK;
+      }
       MfmaCfg c;
       MfmaSplit sp;
       int m_first = m;

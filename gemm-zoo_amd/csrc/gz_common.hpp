@@ -73,8 +73,14 @@ template <> struct Traits<GZ_E5M2E5M2F16> {
   static constexpr bool is_int = false;
 };
 
+// 16-bit running sums (the reference kernels' own accumulators, opt-in): bf16 in chunks of 16 k, fp16 in chunks of 8
+template <> struct Traits<GZ_BF16BF16BF16_ACC16> : Traits<GZ_BF16BF16BF16> {};
+template <> struct Traits<GZ_F16F16F16_ACC16> : Traits<GZ_F16F16F16> {};
+constexpr bool is_acc16(int types) { return types == GZ_BF16BF16BF16_ACC16 || types == GZ_F16F16F16_ACC16; }
+constexpr int acc16_chunk(int types) { return types == GZ_BF16BF16BF16_ACC16 ? 16 : types == GZ_F16F16F16_ACC16 ? 8 : 0; }
+
 constexpr bool is_fp8(int types) { return types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16; }
-constexpr bool out_is_f16(int types) { return types == GZ_F16F16F16 || is_fp8(types); }
+constexpr bool out_is_f16(int types) { return types == GZ_F16F16F16 || types == GZ_F16F16F16_ACC16 || is_fp8(types); }
 
 template <int TYPES> struct GemmArgs {
   using T = Traits<TYPES>;
@@ -151,13 +157,13 @@ template <int TYPES> __host__ __device__ inline typename Traits<TYPES>::acc_t wi
   if constexpr (TYPES == GZ_S8S8S32) return (int32_t)v;
   else if constexpr (TYPES == GZ_E4M3E4M3F16) return e4m3_to_f32(v);
   else if constexpr (TYPES == GZ_E5M2E5M2F16) return e5m2_to_f32(v);
-  else if constexpr (TYPES == GZ_F16F16F16) return f16_to_f32(v);
+  else if constexpr (TYPES == GZ_F16F16F16 || TYPES == GZ_F16F16F16_ACC16) return f16_to_f32(v);
   else if constexpr (TYPES == GZ_F32F32F32) return v;
   else return bf16_to_f32(v);
 }
 
 template <int TYPES> __host__ __device__ inline float round_out(float v) {
-  if constexpr (TYPES == GZ_BF16BF16BF16) return bf16_to_f32(f32_to_bf16(v));
+  if constexpr (TYPES == GZ_BF16BF16BF16 || TYPES == GZ_BF16BF16BF16_ACC16) return bf16_to_f32(f32_to_bf16(v));
   else if constexpr (out_is_f16(TYPES)) return f16_to_f32(f32_to_f16(v));
   else return v;
 }
@@ -181,7 +187,18 @@ __device__ inline typename Traits<TYPES>::out_t epilogue(typename Traits<TYPES>:
     float v = mul_rn(acc, alpha);
     if (beta != 0.0f) v = add_rn(v, mul_rn(beta, *c_ptr));
     return v;
-  } else if constexpr (TYPES == GZ_BF16BF16BF16) {
+  } else if constexpr (TYPES == GZ_F16F16F16_ACC16) {
+    // nvidia/kernels/sm_80/fp16_mma_gemm.cuh:279-290: mul.f16x2 beta * c, then fma.rn.f16x2 alpha * acc + that;
+    // acc, alpha and beta hold fp16 values, so the conversions down are exact and v_fma_f16 rounds once
+    _Float16 bc = (_Float16)0.0f;
+    if (beta != 0.0f) {
+      float q = mul_rn(beta, f16_to_f32(*c_ptr));
+      asm("" : "+v"(q));
+      bc = (_Float16)q;
+    }
+    const _Float16 d = __builtin_fmaf16((_Float16)alpha, (_Float16)acc, bc);
+    return __builtin_bit_cast(uint16_t, d);
+  } else if constexpr (TYPES == GZ_BF16BF16BF16 || TYPES == GZ_BF16BF16BF16_ACC16) {
     float v = round_out<TYPES>(acc);
     v = round_out<TYPES>(mul_rn(v, alpha));
     if (beta != 0.0f) {
@@ -205,6 +222,38 @@ __device__ inline typename Traits<TYPES>::out_t epilogue(typename Traits<TYPES>:
     return f32_to_f16(v);
   }
 }
+
+// 16-bit running sums on the scalar rungs: `part` collects the exact products of one chunk in fp32, in k order; at the
+// chunk's last k it is folded into `acc`, which holds a value of the output type.  k and k_end (the first k that
+// does not exist) count from the same origin, a multiple of the chunk; elements past k_end that a kernel zero-fills
+// add exact zeros, and a chunk made of such elements only is not folded (it would turn a running sum of -0 into +0).
+// Types with an fp32 / int32 accumulator use `acc` alone.  finish() folds a last, shorter chunk.
+template <int TYPES> struct RunningSum {
+  using acc_t = typename Traits<TYPES>::acc_t;
+  acc_t acc = 0, part = 0;
+  __device__ inline void mac(acc_t a, acc_t b, int k, int k_end) {
+    if constexpr (Traits<TYPES>::is_int) {
+      acc += a * b;
+    } else if constexpr (!is_acc16(TYPES)) {
+      acc = __builtin_fmaf(a, b, acc);  // a*b is exact in fp32 for 8- and 16-bit inputs; fp32 inputs: fused by definition
+    } else {
+      part = __builtin_fmaf(a, b, part);
+      if ((k & (acc16_chunk(TYPES) - 1)) == acc16_chunk(TYPES) - 1 && k - (acc16_chunk(TYPES) - 1) < k_end) fold();
+    }
+  }
+  __device__ inline void fold() {
+    if constexpr (is_acc16(TYPES)) {
+      acc = round_out<TYPES>(add_rn(acc, part));
+      part = 0;
+    }
+  }
+  __device__ inline acc_t finish(int k_done) {   // k_done: one past the last k handed to mac()
+    if constexpr (is_acc16(TYPES)) {
+      if (k_done & (acc16_chunk(TYPES) - 1)) fold();
+    }
+    return acc;
+  }
+};
 
 // Same epilogue on an already-loaded C value (for vectorised C loads).
 template <int TYPES>

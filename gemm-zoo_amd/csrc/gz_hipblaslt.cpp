@@ -69,6 +69,10 @@ int gz_hipblaslt_create(int types, int64_t M, int64_t N, int64_t K, int layoutA,
     set_err("gz_hipblaslt_create: bad argument");
     return GZ_ERR_BAD_ARG;
   }
+  if (types == GZ_BF16BF16BF16_ACC16 || types == GZ_F16F16F16_ACC16) {
+    set_err("gz_hipblaslt_create: the library has no 16-bit accumulation");
+    return GZ_ERR_UNSUPPORTED;
+  }
   hipDataType in_t, out_t, scale_t;
   hipblasComputeType_t comp;
   switch (types) {

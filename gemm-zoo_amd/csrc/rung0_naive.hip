@@ -1,27 +1,26 @@
 // Rung 0: one thread per output element, scalar loads, sequential k.
 // Follows the definition of the operation in gemm-zoo
 // (nvidia/kernels/naive_gemm.cuh:6-21, intel/utils/reference_kernel.hpp:12-28),
-// generalised to column-major operands; the accumulator is fp32 / int32.
+// generalised to column-major operands; the accumulator is fp32 / int32, or the 16-bit
+// running sum of the reference's own kernels for the two opt-in modes.
 #include "gz_common.hpp"
 
 namespace gz {
 
 template <int TYPES, bool A_ROW, bool B_ROW>
 __global__ void __launch_bounds__(1024) naive_gemm_kernel(GemmArgs<TYPES> g) {
-  using T = Traits<TYPES>;
   const int col = threadIdx.x + blockIdx.x * blockDim.x;
   const int row = threadIdx.y + blockIdx.y * blockDim.y;
   if (row >= g.M || col >= g.N) return;
 
-  typename T::acc_t acc = 0;
+  RunningSum<TYPES> sum;
   for (int i = 0; i < g.K; i++) {
     const auto a = widen_in<TYPES>(A_ROW ? g.A[(size_t)row * g.K + i] : g.A[(size_t)i * g.M + row]);
     const auto b = widen_in<TYPES>(B_ROW ? g.B[(size_t)i * g.N + col] : g.B[(size_t)col * g.K + i]);
-    if constexpr (T::is_int) acc += a * b;
-    else acc = __builtin_fmaf(a, b, acc);  // a*b is exact in fp32 for 16-bit inputs; fp32 inputs: fused by definition
+    sum.mac(a, b, i, g.K);
   }
   const size_t o = (size_t)row * g.N + col;
-  g.D[o] = epilogue<TYPES>(acc, g.alpha, g.beta, g.C + o);
+  g.D[o] = epilogue<TYPES>(sum.finish(g.K), g.alpha, g.beta, g.C + o);
 }
 
 template <int TYPES> int launch_naive(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
@@ -51,5 +50,7 @@ template int launch_naive<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hipS
 template int launch_naive<GZ_F32F32F32>(const GemmArgs<GZ_F32F32F32>&, int, hipStream_t);
 template int launch_naive<GZ_E4M3E4M3F16>(const GemmArgs<GZ_E4M3E4M3F16>&, int, hipStream_t);
 template int launch_naive<GZ_E5M2E5M2F16>(const GemmArgs<GZ_E5M2E5M2F16>&, int, hipStream_t);
+template int launch_naive<GZ_BF16BF16BF16_ACC16>(const GemmArgs<GZ_BF16BF16BF16_ACC16>&, int, hipStream_t);
+template int launch_naive<GZ_F16F16F16_ACC16>(const GemmArgs<GZ_F16F16F16_ACC16>&, int, hipStream_t);
 
 }  // namespace gz

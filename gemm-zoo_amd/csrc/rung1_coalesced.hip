@@ -26,9 +26,7 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
   const int m0 = blockIdx.y * 16 + (threadIdx.x >> 6) * TM;
   const int n_ld = min(n, N - 1);  // clamped lanes compute a value nobody stores
 
-  acc_t acc[TM];
-#pragma unroll
-  for (int r = 0; r < TM; r++) acc[r] = 0;
+  RunningSum<TYPES> sum[TM];
 
   // 128-bit loads need every line start on a 16-byte boundary
   const bool a_vec = A_KC && (K % EPV == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15u) == 0);
@@ -74,8 +72,7 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
 #pragma unroll
       for (int r = 0; r < TM; r++) {
         const acc_t a = widen_in<TYPES>(av[r][e]);
-        if constexpr (T::is_int) acc[r] += a * b;
-        else acc[r] = __builtin_fmaf(a, b, acc[r]);
+        sum[r].mac(a, b, k0 + e, K);
       }
     }
   }
@@ -86,7 +83,7 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
       const int m = m0 + r;
       if (m < M) {
         const size_t o = (size_t)m * N + n;
-        g.D[o] = epilogue<TYPES>(acc[r], g.alpha, g.beta, g.C + o);
+        g.D[o] = epilogue<TYPES>(sum[r].finish((K + EPV - 1) / EPV * EPV), g.alpha, g.beta, g.C + o);
       }
     }
   }
@@ -118,5 +115,7 @@ template int launch_coalesced<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, 
 template int launch_coalesced<GZ_F32F32F32>(const GemmArgs<GZ_F32F32F32>&, int, hipStream_t);
 template int launch_coalesced<GZ_E4M3E4M3F16>(const GemmArgs<GZ_E4M3E4M3F16>&, int, hipStream_t);
 template int launch_coalesced<GZ_E5M2E5M2F16>(const GemmArgs<GZ_E5M2E5M2F16>&, int, hipStream_t);
+template int launch_coalesced<GZ_BF16BF16BF16_ACC16>(const GemmArgs<GZ_BF16BF16BF16_ACC16>&, int, hipStream_t);
+template int launch_coalesced<GZ_F16F16F16_ACC16>(const GemmArgs<GZ_F16F16F16_ACC16>&, int, hipStream_t);
 
 }  // namespace gz

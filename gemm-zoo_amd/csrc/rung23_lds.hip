@@ -90,15 +90,11 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
   SlabLoader<TYPES, A_KC> la;
   SlabLoader<TYPES, B_KC> lb;
 
-  acc_t acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = 0;
+  RunningSum<TYPES> sum[4][4];
 
   const int slabs = (K + LT_BK - 1) / LT_BK;
 
-  auto compute = [&](const acc_t* as, const acc_t* bs) {
+  auto compute = [&](const acc_t* as, const acc_t* bs, int k_left) {   // k_left: K minus the slab's first k
 #pragma unroll 8
     for (int k = 0; k < LT_BK; k++) {
       const acc4_t a = *reinterpret_cast<const acc4_t*>(as + k * LT_PITCH + ty * 4);
@@ -107,8 +103,7 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
       for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-          if constexpr (T::is_int) acc[i][j] += a[i] * b[j];
-          else acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
+          sum[i][j].mac(a[i], b[j], k, k_left);  // slabs are whole chunks of the 16-bit running sums
         }
     }
   };
@@ -120,7 +115,7 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
       la.store(lds, tid);
       lb.store(lds + SLAB, tid);
       __syncthreads();
-      compute(lds, lds + SLAB);
+      compute(lds, lds + SLAB, K - t * LT_BK);
       __syncthreads();
     }
   } else {
@@ -139,7 +134,7 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
         la.load(g.A, M, K, m0, (t + 1) * LT_BK, tid, a_vec);
         lb.load(g.B, N, K, n0, (t + 1) * LT_BK, tid, b_vec);
       }
-      compute(cur, cur + SLAB);
+      compute(cur, cur + SLAB, K - t * LT_BK);
       if (more) {
         la.store(nxt, tid);
         lb.store(nxt + SLAB, tid);
@@ -157,7 +152,7 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
       const int n = n0 + tx * 4 + j;
       if (n < N) {
         const size_t o = (size_t)m * N + n;
-        g.D[o] = epilogue<TYPES>(acc[i][j], g.alpha, g.beta, g.C + o);
+        g.D[o] = epilogue<TYPES>(sum[i][j].finish(0), g.alpha, g.beta, g.C + o);
       }
     }
   }
@@ -199,6 +194,8 @@ GZ_INST(GZ_F16F16F16)
 GZ_INST(GZ_F32F32F32)
 GZ_INST(GZ_E4M3E4M3F16)
 GZ_INST(GZ_E5M2E5M2F16)
+GZ_INST(GZ_BF16BF16BF16_ACC16)
+GZ_INST(GZ_F16F16F16_ACC16)
 #undef GZ_INST
 
 }  // namespace gz

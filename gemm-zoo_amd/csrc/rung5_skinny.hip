@@ -538,9 +538,9 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
 }
 
 template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
-  if constexpr (TYPES == GZ_S8S8S32 || TYPES == GZ_F32F32F32 || is_fp8(TYPES)) {
+  if constexpr (TYPES == GZ_S8S8S32 || TYPES == GZ_F32F32F32 || is_fp8(TYPES) || is_acc16(TYPES)) {
     (void)g; (void)variant; (void)s;
-    set_error("skinny rung is built for the 16-bit float types only");
+    set_error("skinny rung is built for the 16-bit float types with fp32 accumulation only");
     return GZ_ERR_UNSUPPORTED;
   } else {
     if (variant > 1) {
@@ -588,5 +588,7 @@ template int launch_skinny<GZ_F16F16F16>(const GemmArgs<GZ_F16F16F16>&, int, hip
 template int launch_skinny<GZ_F32F32F32>(const GemmArgs<GZ_F32F32F32>&, int, hipStream_t);
 template int launch_skinny<GZ_E4M3E4M3F16>(const GemmArgs<GZ_E4M3E4M3F16>&, int, hipStream_t);
 template int launch_skinny<GZ_E5M2E5M2F16>(const GemmArgs<GZ_E5M2E5M2F16>&, int, hipStream_t);
+template int launch_skinny<GZ_BF16BF16BF16_ACC16>(const GemmArgs<GZ_BF16BF16BF16_ACC16>&, int, hipStream_t);
+template int launch_skinny<GZ_F16F16F16_ACC16>(const GemmArgs<GZ_F16F16F16_ACC16>&, int, hipStream_t);
 
 }  // namespace gz

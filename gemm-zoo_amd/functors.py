@@ -19,7 +19,10 @@ ROW, COL = capi.ROW_MAJOR, capi.COL_MAJOR
 # (TIn, TOut) -> type bundle, spelled as in the reference's drivers
 BUNDLES = {("s8", "s32"): capi.S8S8S32, ("bf16", "f32"): capi.BF16BF16F32, ("bf16", "bf16"): capi.BF16BF16BF16,
            ("f16", "f16"): capi.F16F16F16, ("f32", "f32"): capi.F32F32F32,
-           ("e4m3", "f16"): capi.E4M3E4M3F16, ("e5m2", "f16"): capi.E5M2E5M2F16}
+           ("e4m3", "f16"): capi.E4M3E4M3F16, ("e5m2", "f16"): capi.E5M2E5M2F16,
+           # the reference kernels' own 16-bit running sums (intel/kernels/xe_gemm_bf16_bf16_bf16_m8k16.hpp:88-107,
+           # nvidia/kernels/sm_80/fp16_mma_gemm.cuh:179,279-290) instead of fp32 accumulation
+           ("bf16", "bf16_acc16"): capi.BF16BF16BF16_ACC16, ("f16", "f16_acc16"): capi.F16F16F16_ACC16}
 
 # functor name -> (rung, tile ints -> variant)
 _RUNGS = {

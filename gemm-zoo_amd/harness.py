@@ -31,19 +31,23 @@ def _torch_types(types):
 
     tin = {capi.S8S8S32: torch.int8, capi.BF16BF16F32: torch.bfloat16, capi.BF16BF16BF16: torch.bfloat16,
            capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32,
-           capi.E4M3E4M3F16: torch.float8_e4m3fn, capi.E5M2E5M2F16: torch.float8_e5m2}[types]
+           capi.E4M3E4M3F16: torch.float8_e4m3fn, capi.E5M2E5M2F16: torch.float8_e5m2,
+           capi.BF16BF16BF16_ACC16: torch.bfloat16, capi.F16F16F16_ACC16: torch.float16}[types]
     tout = {capi.S8S8S32: torch.int32, capi.BF16BF16F32: torch.float32, capi.BF16BF16BF16: torch.bfloat16,
             capi.F16F16F16: torch.float16, capi.F32F32F32: torch.float32,
-            capi.E4M3E4M3F16: torch.float16, capi.E5M2E5M2F16: torch.float16}[types]
+            capi.E4M3E4M3F16: torch.float16, capi.E5M2E5M2F16: torch.float16,
+            capi.BF16BF16BF16_ACC16: torch.bfloat16, capi.F16F16F16_ACC16: torch.float16}[types]
     return tin, tout
 
 
 _IN_DT = {capi.S8S8S32: capi.DT_INT8, capi.BF16BF16F32: capi.DT_BF16, capi.BF16BF16BF16: capi.DT_BF16,
           capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32,
-          capi.E4M3E4M3F16: capi.DT_E4M3, capi.E5M2E5M2F16: capi.DT_E5M2}
+          capi.E4M3E4M3F16: capi.DT_E4M3, capi.E5M2E5M2F16: capi.DT_E5M2,
+          capi.BF16BF16BF16_ACC16: capi.DT_BF16, capi.F16F16F16_ACC16: capi.DT_F16}
 _OUT_DT = {capi.S8S8S32: capi.DT_INT32, capi.BF16BF16F32: capi.DT_F32, capi.BF16BF16BF16: capi.DT_BF16,
            capi.F16F16F16: capi.DT_F16, capi.F32F32F32: capi.DT_F32,
-           capi.E4M3E4M3F16: capi.DT_F16, capi.E5M2E5M2F16: capi.DT_F16}
+           capi.E4M3E4M3F16: capi.DT_F16, capi.E5M2E5M2F16: capi.DT_F16,
+           capi.BF16BF16BF16_ACC16: capi.DT_BF16, capi.F16F16F16_ACC16: capi.DT_F16}
 
 
 def benchmark_impl(kernel_cls, m, n, k, alpha, beta, stream=None, num_repititions=50, verify=True, quiet=False):
@@ -82,6 +86,12 @@ def benchmark_impl(kernel_cls, m, n, k, alpha, beta, stream=None, num_repitition
             fb(m, n, k)(a_s[0], b_s[0], c_s[0], d_ref, alpha, beta, stream)
         if types == capi.S8S8S32:
             thr, rel = 0.0, 0.0
+        elif types in (capi.BF16BF16BF16_ACC16, capi.F16F16F16_ACC16):
+            # two summation orders of a 16-bit running sum part ways by one spacing of the type (at the size the sum
+            # has then, about sqrt(k), up to 4-5 times that among 2^24 outputs) wherever a chunk sum's last fp32
+            # bits move a rounding; a few such events per output are allowed
+            eps = 2.0 ** -8 if types == capi.BF16BF16BF16_ACC16 else 2.0 ** -11
+            thr, rel = 8 * eps * 5 * math.sqrt(k), 1e-2
         elif capi.OUT_SIZE[types] == 2:
             thr, rel = 1e-2 * math.sqrt(k), 1e-2
         else:

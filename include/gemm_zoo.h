@@ -42,6 +42,15 @@
  *                 448; e5m2: the upper byte of an IEEE half); every product is exact in fp32; fp32 accumulate;
  *                 epilogue in fp16 as for f16f16f16 (the reference's checker computes these types in float,
  *                 nvidia/kernels/generic_gemm.cuh:10-13,53-58).
+ *   bf16bf16bf16_acc16, f16f16f16_acc16 : opt-in modes with the reference kernels' 16-bit accumulator.  K is cut into
+ *                 chunks of 16 (bf16: one DPAS of intel/kernels/xe_gemm_bf16_bf16_bf16_m8k16.hpp:88-97, whose C
+ *                 operand is bf16) or 8 (fp16: one mma.sync.m16n8k8.f16.f16.f16.f16 of
+ *                 nvidia/kernels/sm_80/fp16_mma_gemm.cuh:179) consecutive k; a chunk's products are summed in fp32
+ *                 starting from zero, and the 16-bit running sum becomes T(fp32(sum16 + chunk)).  Epilogue bf16:
+ *                 T(T(alpha*acc) + T(beta*C)) (xe_gemm_bf16_bf16_bf16_m8k16.hpp:104-107); fp16: one fused
+ *                 multiply-add in half precision, fma(alpha, acc, T(beta*C)) (fp16_mma_gemm.cuh:279-290).  With
+ *                 beta == 0, C is not read and the addend is +0.  How the hardware of the reference sums inside
+ *                 one instruction is not published; the chunking and the 16-bit running sum are what is modelled.
  *   f32f32f32   : fp32 accumulate in k order with each product fused into the sum (fma), which is what the
  *                 reference's `acc += a * b` (nvidia/kernels/naive_gemm.cuh:16-19) compiles to; epilogue as
  *                 bf16bf16f32.  The MFMA rung uses the full-precision v_mfma_f32_32x32x2_f32, not a tf32 mode.
@@ -74,7 +83,9 @@ typedef enum gz_types {
   GZ_F32F32F32 = 4,
   GZ_E4M3E4M3F16 = 5, /* OCP fp8 e4m3 (finite-only, __nv_fp8_e4m3's format) x e4m3 -> fp16 */
   GZ_E5M2E5M2F16 = 6, /* OCP fp8 e5m2 (__nv_fp8_e5m2's format) x e5m2 -> fp16            */
-  GZ_NUM_TYPES = 7
+  GZ_BF16BF16BF16_ACC16 = 7, /* bf16 x bf16 -> bf16 with a bf16 running sum, chunks of 16 k */
+  GZ_F16F16F16_ACC16 = 8,    /* fp16 x fp16 -> fp16 with an fp16 running sum, chunks of 8 k  */
+  GZ_NUM_TYPES = 9
 } gz_types;
 
 /* The ladder.  GZ_RUNG_AUTO lets the launcher pick (MFMA, or the weight-streaming
@@ -144,6 +155,18 @@ int gz_gemm_e4m3e4m3f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, u
 int gz_gemm_e5m2e5m2f16(const uint8_t* A, const uint8_t* B, const uint16_t* C, uint16_t* D,
                         int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                         float alpha, float beta, int rung, int variant, gz_stream stream);
+
+/* The reference kernels' own 16-bit accumulators as opt-in modes (see the arithmetic contract above): the bf16
+ * accumulator of intel::gemm_bf16_bf16_bf16_m8k16 (intel/kernels/xe_gemm_bf16_bf16_bf16_m8k16.hpp:88-107) and the
+ * fp16 accumulator of nvidia::kernels::sm80::fp16_mma_gemm (nvidia/kernels/sm_80/fp16_mma_gemm.cuh:179,279-290).
+ * Served by the naive, coalesced, LDS-tiled, double-buffered and MFMA rungs; the weight-streaming rung refuses.  */
+int gz_gemm_bf16bf16bf16_acc16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                               int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                               float alpha, float beta, int rung, int variant, gz_stream stream);
+
+int gz_gemm_f16f16f16_acc16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                            int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                            float alpha, float beta, int rung, int variant, gz_stream stream);
 
 /* Type-erased form of the typed entry points above (alpha/beta as double; for s8s8s32 they must be
  * integral).                                                                         */

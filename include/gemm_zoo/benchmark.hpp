@@ -46,6 +46,8 @@ template <typename T> struct elem;  // gz_fill / gz_compare element codes
 template <> struct elem<int8_t> { static constexpr int dt = 0, kind = 0; };
 template <> struct elem<gemm_zoo::bf16_t> { static constexpr int dt = 1, kind = 1; };
 template <> struct elem<gemm_zoo::half_t> { static constexpr int dt = 2, kind = 1; };
+template <> struct elem<gemm_zoo::bf16_acc16_t> { static constexpr int dt = 1, kind = 1; };
+template <> struct elem<gemm_zoo::half_acc16_t> { static constexpr int dt = 2, kind = 1; };
 template <> struct elem<float> { static constexpr int dt = 3, kind = 1; };
 template <> struct elem<int32_t> { static constexpr int dt = 4, kind = 0; };
 template <> struct elem<gemm_zoo::e4m3_t> { static constexpr int dt = 5, kind = 1; };
@@ -103,10 +105,15 @@ result benchmark_impl(std::size_t m, std::size_t n, std::size_t k, TOut alpha, T
     float threshold = 0.5f, relative = 0.0f;
     if constexpr (std::is_same_v<TOut, int32_t>) threshold = 0.0f;
     else if constexpr (sizeof(TOut) == 2) { threshold = 1e-2f * std::sqrt((float)k); relative = 1e-2f; }
+    // 16-bit running sums: two summation orders part ways wherever a chunk sum's last fp32 bits move a rounding of
+    // the running sum, by one spacing of the 16-bit type at the size the sum has then (about sqrt(k), up to 4-5
+    // times that in 2^24 outputs); a few such events per output are allowed
+    if constexpr (std::is_same_v<TOut, gemm_zoo::half_acc16_t>) threshold = 8.0f * 0x1p-11f * 5.0f * std::sqrt((float)k);
+    if constexpr (std::is_same_v<TOut, gemm_zoo::bf16_acc16_t>) threshold = 8.0f * 0x1p-8f * 5.0f * std::sqrt((float)k);
     int64_t different = 0;
     const int st = gz_compare_rel(d_out, d_ref, (int64_t)(m * n), elem<TOut>::dt, threshold, relative, &different,
                                   stream);
-    if (st != GZ_OK) throw std::runtime_error("verification failed");
+    if (st != GZ_OK) throw std::runtime_error(std::string("verification failed: ") + gz_last_error());
   }
 
   hipEvent_t start, stop;
@@ -170,8 +177,8 @@ template <class Kernel, typename TIn, typename TOut, gemm_zoo::layout LA = gemm_
 void benchmark_sizes(const std::vector<std::tuple<std::size_t, std::size_t, std::size_t>>& sizes, hipStream_t stream,
                      const int num_repititions = 50) {
   TOut alpha, beta;
-  if constexpr (std::is_same_v<TOut, gemm_zoo::bf16_t>) { alpha.bits = beta.bits = 0x3F80; }
-  else if constexpr (std::is_same_v<TOut, gemm_zoo::half_t>) { alpha.bits = beta.bits = 0x3C00; }
+  if constexpr (std::is_same_v<TOut, gemm_zoo::bf16_t> || std::is_same_v<TOut, gemm_zoo::bf16_acc16_t>) { alpha.bits = beta.bits = 0x3F80; }
+  else if constexpr (std::is_same_v<TOut, gemm_zoo::half_t> || std::is_same_v<TOut, gemm_zoo::half_acc16_t>) { alpha.bits = beta.bits = 0x3C00; }
   else { alpha = beta = static_cast<TOut>(1); }
   for (const auto& [m, n, k] : sizes)
     detail::benchmark_impl<Kernel, TIn, TOut, LA, LB>(m, n, k, alpha, beta, stream, num_repititions);

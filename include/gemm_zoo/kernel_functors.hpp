@@ -30,6 +30,11 @@ namespace gemm_zoo {
 // 16-bit storage types (bit patterns); enough for hosts that only move data around.
 struct bf16_t { uint16_t bits; };
 struct half_t { uint16_t bits; };
+// Output types that also ask for the reference kernels' own 16-bit running sum instead of fp32 accumulation
+// (bf16: intel/kernels/xe_gemm_bf16_bf16_bf16_m8k16.hpp:88-107; fp16: nvidia/kernels/sm_80/fp16_mma_gemm.cuh:179,
+// 279-290): same storage as bf16_t / half_t, e.g. fp16_mma_gemm<half_t, half_acc16_t>.
+struct bf16_acc16_t { uint16_t bits; };
+struct half_acc16_t { uint16_t bits; };
 // OCP 8-bit floats (the formats of __nv_fp8_e4m3 / __nv_fp8_e5m2), inputs only
 struct e4m3_t { uint8_t bits; };
 struct e5m2_t { uint8_t bits; };
@@ -44,12 +49,16 @@ inline float to_float(bf16_t v) { return bits_to_float((uint32_t)v.bits << 16); 
 inline float to_float(half_t v) {
   _Float16 h; __builtin_memcpy(&h, &v.bits, 2); return (float)h;
 }
+inline float to_float(bf16_acc16_t v) { return to_float(bf16_t{v.bits}); }
+inline float to_float(half_acc16_t v) { return to_float(half_t{v.bits}); }
 
 template <typename TIn, typename TOut> struct bundle;  // (TIn, TOut) -> gz_types
 template <> struct bundle<int8_t, int32_t> { static constexpr int value = GZ_S8S8S32; };
 template <> struct bundle<bf16_t, float> { static constexpr int value = GZ_BF16BF16F32; };
 template <> struct bundle<bf16_t, bf16_t> { static constexpr int value = GZ_BF16BF16BF16; };
 template <> struct bundle<half_t, half_t> { static constexpr int value = GZ_F16F16F16; };
+template <> struct bundle<bf16_t, bf16_acc16_t> { static constexpr int value = GZ_BF16BF16BF16_ACC16; };
+template <> struct bundle<half_t, half_acc16_t> { static constexpr int value = GZ_F16F16F16_ACC16; };
 template <> struct bundle<float, float> { static constexpr int value = GZ_F32F32F32; };  // the reference's ladder drivers
 // nvidia/bench/bench_cublaslt_e4m3.cu:9-11, bench_cublaslt_e5m2.cu:9-11
 template <> struct bundle<e4m3_t, half_t> { static constexpr int value = GZ_E4M3E4M3F16; };
@@ -150,11 +159,13 @@ struct bf16_mma_gemm : detail::functor_base<TIn, TOut, LA, LB> {
   GZ_FUNCTOR_COMMON(bf16_mma_gemm, GZ_RUNG_MFMA, detail::mfma_variant_for(M, N))
 };
 
-// nvidia/kernel_functors/fp16_mma_gemm.cuh:16-70 (fp16 x fp16 -> fp16, fp32 accumulate here)
+// nvidia/kernel_functors/fp16_mma_gemm.cuh:16-70 (fp16 x fp16 -> fp16; fp32 accumulate with TOut = half_t, the
+// reference's fp16 accumulate with TOut = half_acc16_t)
 template <typename TIn, typename TOut, int M = 256, int N = 256, int K = 64, layout LA = layout::row_major,
           layout LB = layout::row_major>
 struct fp16_mma_gemm : detail::functor_base<TIn, TOut, LA, LB> {
-  static_assert(std::is_same_v<TIn, half_t> && std::is_same_v<TOut, half_t>, "fp16 in and out");
+  static_assert(std::is_same_v<TIn, half_t> && (std::is_same_v<TOut, half_t> || std::is_same_v<TOut, half_acc16_t>),
+                "fp16 in and out");
   GZ_FUNCTOR_COMMON(fp16_mma_gemm, GZ_RUNG_MFMA, detail::mfma_variant_for(M, N))
 };
 

@@ -29,6 +29,14 @@
  *     (OCP 8-bit Floating Point Specification v1.0): e4m3 = 1-4-3 bits, bias 7, no infinities, S.1111.111 NaN,
  *     largest finite 448; e5m2 = 1-5-2 bits, bias 15, IEEE-style infinities and NaNs.   -> oracle_fp8_*()
  *
+ *   - the 16-bit accumulators of intel/kernels/xe_gemm_bf16_bf16_bf16_m8k16.hpp:88-107 (bf16 C operand of every
+ *     DPAS, bf16 epilogue) and nvidia/kernels/sm_80/fp16_mma_gemm.cuh:179,279-290 (fp16 C operand of every
+ *     mma.sync.m16n8k8, mul.f16x2 / fma.rn.f16x2 epilogue) as the bundles *_ACC16: chunks of 16 / 8 k, fp32 inside
+ *     a chunk, the running sum rounded to 16 bits after every chunk (see store_acc16 and the comment above it).
+ *     What the two devices do inside one instruction is not published and the reference holds no output of
+ *     these kernels: the model is pinned as arithmetic (below), its agreement with either device is
+ *     PARITY UNPINNED.
+ *
  *   - layouts: the reference only knows row-major operands; column-major A/B
  *     is the generalisation  A(i,p) = rowmajor ? a[i*K+p] : a[p*M+i].
  *
@@ -52,6 +60,12 @@
  *                         encode(decode(code)) == code, ties-to-even and saturation known answers; the GEMM
  *                         on fp8 inputs against exact integer arithmetic (every product and partial sum of
  *                         small codes is exact) and fp64 truth.
+ *   *_ACC16 bundles       closed forms that separate a 16-bit running sum from an fp32 one and one chunk length
+ *                         from another (K ones stop growing at 4096 for bf16 / 16, at 16384 for fp16 / 8), an
+ *                         independent model in numpy (float32 adds, numpy float16 / torch bfloat16 roundings),
+ *                         oracle_f64_to_f16 against numpy on every fp16 value, its midpoints and neighbours,
+ *                         oracle_fma_f16 against exact rational arithmetic incl. a product on a rounding tie
+ *                         that a tiny addend must break (fails any two-step multiply-add).
  *   bf16/fp16 converters  closed-form RNE known answers, exhaustive 2^16
  *                         round trips, numpy float16 / torch bfloat16.
  *   philox4x32_10         Random123 known-answer vectors.
@@ -71,7 +85,7 @@
 #define ORACLE_API __attribute__((visibility("default")))
 
 enum { OR_S8S8S32 = 0, OR_BF16BF16F32 = 1, OR_BF16BF16BF16 = 2, OR_F16F16F16 = 3, OR_F32F32F32 = 4,
-       OR_E4M3E4M3F16 = 5, OR_E5M2E5M2F16 = 6, OR_NUM_TYPES = 7 };
+       OR_E4M3E4M3F16 = 5, OR_E5M2E5M2F16 = 6, OR_BF16BF16BF16_ACC16 = 7, OR_F16F16F16_ACC16 = 8, OR_NUM_TYPES = 9 };
 enum { OR_ROW = 0, OR_COL = 1 };
 
 /* ------------------------------------------------------------------------ */
@@ -171,10 +185,74 @@ ORACLE_API uint8_t oracle_f32_to_fp8(int e5m2, float f) {
 
 static inline int is_fp8(int types) { return types == OR_E4M3E4M3F16 || types == OR_E5M2E5M2F16; }
 
+static inline int is_acc16(int types) { return types == OR_BF16BF16BF16_ACC16 || types == OR_F16F16F16_ACC16; }
+static inline int out_is_bf16(int types) { return types == OR_BF16BF16BF16 || types == OR_BF16BF16BF16_ACC16; }
+static inline int in_is_f16(int types) { return types == OR_F16F16F16 || types == OR_F16F16F16_ACC16; }
+
 static inline float round_to(int types, float v) {
-  if (types == OR_BF16BF16BF16) return oracle_bf16_to_f32(oracle_f32_to_bf16(v));
-  if (types == OR_F16F16F16 || is_fp8(types)) return oracle_f16_to_f32(oracle_f32_to_f16(v));
+  if (out_is_bf16(types)) return oracle_bf16_to_f32(oracle_f32_to_bf16(v));
+  if (in_is_f16(types) || is_fp8(types)) return oracle_f16_to_f32(oracle_f32_to_f16(v));
   return v;
+}
+
+/* ------------------------------------------------------------------------ */
+/* The reference kernels' 16-bit accumulators (opt-in bundles *_ACC16).      */
+/*   intel/kernels/xe_gemm_bf16_bf16_bf16_m8k16.hpp:88-97: two DPAS per k-tile of 32, 16 k each, with the        */
+/*     SPIRV_MatrixCBf16 flag: the accumulator that goes in and comes out of every instruction is bf16.          */
+/*   nvidia/kernels/sm_80/fp16_mma_gemm.cuh:179: mma.sync.m16n8k8 ... f16.f16.f16.f16, 8 k each, fp16 C and D.   */
+/* How either device sums inside one instruction is not published.  The model: K is cut into chunks of 16        */
+/* (bf16) / 8 (fp16) consecutive k; a chunk's exact products are added in k order in fp32 from zero; the         */
+/* running sum becomes T(fp32(sum + chunk)).  A last, shorter chunk is a chunk like any other.                   */
+/* Epilogues: bf16  d = T(T(alpha*acc) + T(beta*c))  (xe_gemm_bf16_bf16_bf16_m8k16.hpp:104-107: the operators    */
+/*   of sycl's bfloat16 compute in float and round the result), the generic epilogue on an already-bf16 sum;     */
+/*   fp16  d = fma.rn.f16(alpha, acc, mul.f16(beta, c))  (fp16_mma_gemm.cuh:279-290): one rounding for the fused */
+/*   multiply-add.  beta == 0: c is not read, the addend is +0.                                                  */
+/* ------------------------------------------------------------------------ */
+static inline int acc16_chunk(int types) { return types == OR_BF16BF16BF16_ACC16 ? 16 : 8; }
+
+/* double -> fp16, round to nearest even, from the value itself (no intermediate float) */
+ORACLE_API uint16_t oracle_f64_to_f16(double v) {
+  uint64_t bits; memcpy(&bits, &v, 8);
+  const uint16_t sign = (uint16_t)((bits >> 48) & 0x8000u);
+  if (isnan(v)) return (uint16_t)(sign | 0x7e00u);
+  const double a = fabs(v);
+  if (a >= 65520.0) return (uint16_t)(sign | 0x7c00u); /* halfway between 65504 and 2^16 rounds to even = infinity */
+  if (a == 0.0) return sign;
+  int e; (void)frexp(a, &e);          /* a = m 2^e, 0.5 <= m < 1: leading bit 2^(e-1) */
+  int E = e - 1;
+  if (E < -14) E = -14;               /* subnormals share the smallest normal's spacing */
+  const double q = rint(ldexp(a, 10 - E)); /* a in units of 2^(E-10): exact scaling, then nearest-even (default mode) */
+  /* normal: q in [1024, 2048] holds the implicit bit, so ((E+14) << 10) + q; subnormal: E = -14, the code is q;
+   * a carry to 2048 lands in the next binade either way */
+  return (uint16_t)(sign | (uint16_t)(((uint32_t)(E + 14) << 10) + (uint32_t)q));
+}
+
+/* fma.rn.f16: a*b + c rounded once.  a, b, c hold fp16 values, so a*b is exact in double; the sum is exact in double
+ * unless the addends are very far apart, and then the low part (TwoSum) only has to break a tie */
+ORACLE_API uint16_t oracle_fma_f16(float a, float b, float c) {
+  const double p = (double)a * (double)b;
+  double s = p + (double)c;
+  if (isfinite(s)) {
+    const double bb = s - p;
+    const double err = (p - (s - bb)) + ((double)c - bb);
+    if (err > 0) s = nextafter(s, INFINITY);
+    else if (err < 0) s = nextafter(s, -INFINITY);
+  }
+  return oracle_f64_to_f16(s);
+}
+
+/* epilogue of the *_ACC16 bundles on a running sum `acc` that already holds a value of the output type */
+static inline void store_acc16(int types, void* D, const void* C, size_t idx, float acc, float alpha, float beta) {
+  uint16_t* d = (uint16_t*)D;
+  const uint16_t* c = (const uint16_t*)C;
+  if (types == OR_BF16BF16BF16_ACC16) {
+    float val = round_to(types, acc * alpha);
+    if (beta != 0.0f) val = round_to(types, val + round_to(types, beta * oracle_bf16_to_f32(c[idx])));
+    d[idx] = oracle_f32_to_bf16(val);
+  } else {
+    const float bc = beta != 0.0f ? round_to(types, beta * oracle_f16_to_f32(c[idx])) : 0.0f;
+    d[idx] = oracle_fma_f16(alpha, acc, bc);
+  }
 }
 
 /* ------------------------------------------------------------------------ */
@@ -230,18 +308,18 @@ static float load_in_f32(int types, const void* p, size_t idx) {
   if (types == OR_E4M3E4M3F16) return oracle_fp8_to_f32(0, ((const uint8_t*)p)[idx]);
   if (types == OR_E5M2E5M2F16) return oracle_fp8_to_f32(1, ((const uint8_t*)p)[idx]);
   const uint16_t* h = (const uint16_t*)p;
-  return types == OR_F16F16F16 ? oracle_f16_to_f32(h[idx]) : oracle_bf16_to_f32(h[idx]);
+  return in_is_f16(types) ? oracle_f16_to_f32(h[idx]) : oracle_bf16_to_f32(h[idx]);
 }
 
 static float load_out_f32(int types, const void* p, size_t idx) {
   if (types == OR_BF16BF16F32 || types == OR_F32F32F32) return ((const float*)p)[idx];
-  if (types == OR_BF16BF16BF16) return oracle_bf16_to_f32(((const uint16_t*)p)[idx]);
+  if (out_is_bf16(types)) return oracle_bf16_to_f32(((const uint16_t*)p)[idx]);
   return oracle_f16_to_f32(((const uint16_t*)p)[idx]);
 }
 
 static void store_out_f32(int types, void* p, size_t idx, float v) {
   if (types == OR_BF16BF16F32 || types == OR_F32F32F32) ((float*)p)[idx] = v;
-  else if (types == OR_BF16BF16BF16) ((uint16_t*)p)[idx] = oracle_f32_to_bf16(v);
+  else if (out_is_bf16(types)) ((uint16_t*)p)[idx] = oracle_f32_to_bf16(v);
   else ((uint16_t*)p)[idx] = oracle_f32_to_f16(v);
 }
 
@@ -310,14 +388,20 @@ ORACLE_API int oracle_gemm_rows(int types, const void* A, const void* B, const v
 
 #pragma omp parallel num_threads(threads)
   {
-    float* acc = (float*)malloc(sizeof(float) * (size_t)N);
+    float* acc = (float*)malloc(sizeof(float) * (size_t)N * 2);
+    float* part = acc + N;
 #pragma omp for schedule(dynamic, 4)
     for (int64_t i = row0; i < row1; i++) {
-      for (int64_t j = 0; j < N; j++) acc[j] = 0.0f;
+      for (int64_t j = 0; j < N; j++) acc[j] = 0.0f, part[j] = 0.0f;
       for (int64_t p = 0; p < K; p++) {
         const float av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
         const float* brow = bf + p * N;
-        if (types == OR_F32F32F32) {
+        if (is_acc16(types)) {
+          /* 16-bit running sum: the chunk's products in fp32 from zero, folded at the chunk's last k */
+          for (int64_t j = 0; j < N; j++) part[j] = part[j] + av * brow[j];
+          if ((p + 1) % acc16_chunk(types) == 0 || p + 1 == K)
+            for (int64_t j = 0; j < N; j++) acc[j] = round_to(types, acc[j] + part[j]), part[j] = 0.0f;
+        } else if (types == OR_F32F32F32) {
           /* fp32 inputs: the product is fused into the sum, which is what `acc += a * b` of the reference
            * kernels (nvidia/kernels/naive_gemm.cuh:16-19) compiles to under nvcc's and icpx's defaults */
           for (int64_t j = 0; j < N; j++) acc[j] = __builtin_fmaf(av, brow[j], acc[j]);
@@ -325,6 +409,10 @@ ORACLE_API int oracle_gemm_rows(int types, const void* A, const void* B, const v
           /* a*b is exact in fp32 for 16-bit inputs; one rounding per add */
           for (int64_t j = 0; j < N; j++) acc[j] = acc[j] + av * brow[j];
         }
+      }
+      if (is_acc16(types)) {
+        for (int64_t j = 0; j < N; j++) store_acc16(types, D, C, (size_t)(i * N + j), acc[j], alpha, beta);
+        continue;
       }
       for (int64_t j = 0; j < N; j++) {
         /* generic_gemm.cuh:53-58, every operation rounded to TOut */
@@ -385,11 +473,20 @@ ORACLE_API int oracle_gemm_naive_rows(int types, const void* A, const void* B, c
       if (ibeta != 0) v += ibeta * (uint32_t)((const int32_t*)C)[gid];
       ((int32_t*)D)[gid] = (int32_t)v;
     } else {
-      float acc = 0.0f;
+      float acc = 0.0f, part = 0.0f;
       for (int64_t p = 0; p < K; p++) {
         float av = load_in_f32(types, A, layoutA == OR_ROW ? (size_t)(i * K + p) : (size_t)(p * M + i));
         float bv = load_in_f32(types, B, layoutB == OR_ROW ? (size_t)(p * N + j) : (size_t)(j * K + p));
-        acc = types == OR_F32F32F32 ? __builtin_fmaf(av, bv, acc) : acc + av * bv;
+        if (is_acc16(types)) {
+          part = part + av * bv;
+          if ((p + 1) % acc16_chunk(types) == 0 || p + 1 == K) acc = round_to(types, acc + part), part = 0.0f;
+        } else {
+          acc = types == OR_F32F32F32 ? __builtin_fmaf(av, bv, acc) : acc + av * bv;
+        }
+      }
+      if (is_acc16(types)) {
+        store_acc16(types, D, C, (size_t)gid, acc, alpha, beta);
+        continue;
       }
       float val = round_to(types, acc);
       val = round_to(types, val * alpha);

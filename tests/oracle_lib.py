@@ -12,16 +12,21 @@ ORACLE_DIR = ROOT / "oracle"
 LIB = ORACLE_DIR / "liboracle.so"
 
 S8S8S32, BF16BF16F32, BF16BF16BF16, F16F16F16, F32F32F32, E4M3E4M3F16, E5M2E5M2F16 = 0, 1, 2, 3, 4, 5, 6
+BF16BF16BF16_ACC16, F16F16F16_ACC16 = 7, 8   # the reference kernels' 16-bit running sums (chunks of 16 / 8 k)
 FP8_TYPES = (E4M3E4M3F16, E5M2E5M2F16)
+ACC16_TYPES = (BF16BF16BF16_ACC16, F16F16F16_ACC16)
+ACC16_CHUNK = {BF16BF16BF16_ACC16: 16, F16F16F16_ACC16: 8}
 ROW, COL = 0, 1
-IN_DTYPE = {0: np.int8, 1: np.uint16, 2: np.uint16, 3: np.uint16, 4: np.float32, 5: np.uint8, 6: np.uint8}
-OUT_DTYPE = {0: np.int32, 1: np.float32, 2: np.uint16, 3: np.uint16, 4: np.float32, 5: np.uint16, 6: np.uint16}
+IN_DTYPE = {0: np.int8, 1: np.uint16, 2: np.uint16, 3: np.uint16, 4: np.float32, 5: np.uint8, 6: np.uint8, 7: np.uint16,
+            8: np.uint16}
+OUT_DTYPE = {0: np.int32, 1: np.float32, 2: np.uint16, 3: np.uint16, 4: np.float32, 5: np.uint16, 6: np.uint16,
+             7: np.uint16, 8: np.uint16}
 # gz_fill / oracle_fill codes
 DT_INT8, DT_BF16, DT_F16, DT_F32, DT_INT32, DT_E4M3, DT_E5M2 = 0, 1, 2, 3, 4, 5, 6
 NP_OF_DT = {0: np.int8, 1: np.uint16, 2: np.uint16, 3: np.float32, 4: np.int32, 5: np.uint8, 6: np.uint8}
 FILL_INT8_UNIFORM, FILL_NORMAL, FILL_UNIFORM_PM1, FILL_SMALL_INT = 0, 1, 2, 3
-IN_DT = {0: DT_INT8, 1: DT_BF16, 2: DT_BF16, 3: DT_F16, 4: DT_F32, 5: DT_E4M3, 6: DT_E5M2}
-OUT_DT = {0: DT_INT32, 1: DT_F32, 2: DT_BF16, 3: DT_F16, 4: DT_F32, 5: DT_F16, 6: DT_F16}
+IN_DT = {0: DT_INT8, 1: DT_BF16, 2: DT_BF16, 3: DT_F16, 4: DT_F32, 5: DT_E4M3, 6: DT_E5M2, 7: DT_BF16, 8: DT_F16}
+OUT_DT = {0: DT_INT32, 1: DT_F32, 2: DT_BF16, 3: DT_F16, 4: DT_F32, 5: DT_F16, 6: DT_F16, 7: DT_BF16, 8: DT_F16}
 
 
 def _load():
@@ -50,6 +55,10 @@ def _load():
     lib.oracle_fp8_to_f32.restype = C.c_float
     lib.oracle_f32_to_fp8.argtypes = [i32, C.c_float]
     lib.oracle_f32_to_fp8.restype = C.c_uint8
+    lib.oracle_f64_to_f16.argtypes = [C.c_double]
+    lib.oracle_f64_to_f16.restype = C.c_uint16
+    lib.oracle_fma_f16.argtypes = [C.c_float, C.c_float, C.c_float]
+    lib.oracle_fma_f16.restype = C.c_uint16
     lib.oracle_normal_from_words.argtypes = [C.c_uint32, C.c_uint32]
     lib.oracle_normal_from_words.restype = C.c_float
     lib.oracle_num_threads.restype = i32
@@ -111,9 +120,9 @@ def f16_to_f32(bits: np.ndarray) -> np.ndarray:
 
 
 def out_to_f64(types, d: np.ndarray) -> np.ndarray:
-    if types == BF16BF16BF16:
+    if types in (BF16BF16BF16, BF16BF16BF16_ACC16):
         return bf16_to_f32(d).astype(np.float64)
-    if types == F16F16F16 or types in FP8_TYPES:
+    if types in (F16F16F16, F16F16F16_ACC16) or types in FP8_TYPES:
         return f16_to_f32(d).astype(np.float64)
     return d.astype(np.float64)
 

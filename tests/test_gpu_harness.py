@@ -58,6 +58,10 @@ def test_harness_runs_verifies_and_reports(G, capsys):
     for tin in ("e4m3", "e5m2"):
         r = H.benchmark(F.functor("fp8_mma_gemm", tin, "f16"), [(512, 256, 384)], 1.0, 1.0, num_repititions=2)[0]
         assert r.tflops > 0
+    # the reference kernels' own 16-bit running sums, verified against the any-shape rung in the same mode
+    for name, tin, tout in (("fp16_mma_gemm", "f16", "f16_acc16"), ("gemm_bf16_bf16_bf16_m8k16", "bf16", "bf16_acc16")):
+        r = H.benchmark(F.functor(name, tin, tout), [(384, 256, 1024)], 1.0, 1.0, num_repititions=2)[0]
+        assert r.tflops > 0
     S = F.functor("gemm_s8_s8_s32_m8k16", "s8", "s32", layout_b=F.COL)
     r = H.benchmark_sizes(S, [(512, 512, 512)], num_repititions=2)[0]
     assert r.gbps > 0

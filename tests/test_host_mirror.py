@@ -74,4 +74,5 @@ def test_comparator_library_exports(F):
     for n in names:
         assert hasattr(lib, n)
     plan = ctypes.c_void_p()
-    assert lib.gz_hipblaslt_create(7, 4, 4, 4, 0, 0, ctypes.byref(plan)) == 1  # bad type bundle, no device touched
+    assert lib.gz_hipblaslt_create(9, 4, 4, 4, 0, 0, ctypes.byref(plan)) == 1  # bad type bundle, no device touched
+    assert lib.gz_hipblaslt_create(7, 4, 4, 4, 0, 0, ctypes.byref(plan)) == 2  # 16-bit running sums: not in the library
