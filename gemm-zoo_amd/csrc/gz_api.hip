@@ -91,6 +91,7 @@ static int run(const void* A, const void* B, const void* C, void* D, int64_t M, 
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   g.layoutA = layoutA; g.layoutB = layoutB;
   g.alpha = alpha; g.beta = beta;
+  g.store_hint = 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   int resolved = resolve_rung(TYPES, M, N, K, layoutA, layoutB, rung);

@@ -91,6 +91,7 @@ template <int TYPES> struct GemmArgs {
   int M, N, K;
   int layoutA, layoutB;
   typename T::scalar_t alpha, beta;
+  int store_hint;   // MFMA rung: 1 = the stores of D carry the non-temporal hint (set by the launcher)
 };
 
 // ---------------------------------------------------------------------------

@@ -78,6 +78,20 @@ inline int mfma_in_size(int types) {
   return (types == GZ_S8S8S32 || types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) ? 1 : types == GZ_F32F32F32 ? 4 : 2;
 }
 
+// Whether the stores of D carry the non-temporal hint.  Measured in interleaved runs, plain / non-temporal (us):
+// outputs of 64 MiB: bf16 4096 x 4096 x {64, 1024, 4096} 17.9 / 17.5, 43.5 / 42.0, 120.2 / 119.1; several rounds of
+// tiles with a long K, where the writes of one round overlap the next round's loads and no longer push operands out
+// of the caches: bf16 8192^3 867 / 838, int8 8192^3 493.5 / 486.4, fp8 8192^3 415.5 / 413.7.  A launch that is
+// mostly the writing of an output larger than that loses with the hint (int8 8192 x 8192 x {128, 512, 1024, 2048}
+// 65 / 77, 86 / 96, 106 / 115, 158 / 163; bf16 8192 x 8192 x 256 80 / 88): the last-level cache no longer takes the
+// burst in.  In between (6144^2 x 4096, int8 8192^2 x 4096) it makes no difference.
+inline int mfma_store_hint(int types, long long M, long long N, long long K, int out_size, int num_cus) {
+  const long long out_bytes = M * N * out_size;
+  if (out_bytes <= (64ll << 20)) return 1;
+  const long long tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  return (tiles >= 4ll * num_cus && K * mfma_in_size(types) >= 8192) ? 1 : 0;
+}
+
 // The launcher's own choice for one launch over the whole problem; returns the estimate it was chosen by.
 inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaCfg* out) {
   if (num_cus <= 0) num_cus = 256;

@@ -189,7 +189,19 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         dv[1] = epilogue<TYPES>(v[1], g.alpha, g.beta, &cv[T][1]);
         dv[2] = epilogue<TYPES>(v[2], g.alpha, g.beta, &cv[T][2]);
         dv[3] = epilogue<TYPES>(v[3], g.alpha, g.beta, &cv[T][3]);
-        __builtin_memcpy(g.D + o, dv, sizeof(dv));
+        if (g.store_hint) {   // non-temporal: see mfma_store_hint
+          if constexpr (sizeof(out_t) == 4) {
+            u32x4_t w;
+            __builtin_memcpy(&w, dv, 16);
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t*>(g.D + o));
+          } else {
+            u32x2_t w;
+            __builtin_memcpy(&w, dv, 8);
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x2_t*>(g.D + o));
+          }
+        } else {
+          __builtin_memcpy(g.D + o, dv, sizeof(dv));
+        }
       });
     } else if constexpr (RAGGED) {
       for (int r = 0; r < 32; r++) {
@@ -1212,7 +1224,9 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
   return GZ_ERR_UNSUPPORTED;
 }
 
-template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
+template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, hipStream_t s) {
+  GemmArgs<TYPES> g = args;
+  g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), 256);
   if (variant == 0 && g.K > 0) {
     // a mostly empty last round of 256x256 tiles: the rows that fill whole rounds first, the rest in a second launch
     MfmaSplit sp;
