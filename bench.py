@@ -209,9 +209,24 @@ def main() -> int:
         t32 = flops / (r32["kernel_ms_mean"] * 1e-3) / 1e12
         extras["f32_4096_row_row"] = {"tflops": round(t32, 2), "frac_of_f32_peak": round(t32 / PEAK_TFLOPS["f32"], 4),
                                       "kernel_ms_mean": round(r32["kernel_ms_mean"], 5)}
+        # the two remaining configurations of the baseline: int8 1024^3 (row-major A and B) and the ragged fp16
+        # problem 4095 x 4097 x 1023 (row-major A and B, predicated edge tiles, unaligned rows)
+        rs1 = timed(capi.S8S8S32, 1024, 1024, 1024, capi.ROW_MAJOR, capi.ROW_MAJOR, 100, 100)
+        extras["s8_1024_row_row"] = {"tops": round(2.0 * 1024 ** 3 / (rs1["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                                     "kernel_us_mean": round(rs1["kernel_ms_mean"] * 1e3, 2)}
+        rg = timed(capi.F16F16F16, 4095, 4097, 1023, capi.ROW_MAJOR, capi.ROW_MAJOR, 50, 50)
+        extras["f16_4095x4097x1023_row_row"] = {
+            "tflops": round(2.0 * 4095 * 4097 * 1023 / (rg["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+            "kernel_us_mean": round(rg["kernel_ms_mean"] * 1e3, 2)}
         # the vendor library beside it (the reference reports cuBLASLt): same operands, same timing, checked the same way
         try:
             functors = importlib.import_module("gemm-zoo_amd.functors")
+            lt = functors.HipblasLtGemm(capi.F16F16F16, 4095, 4097, 1023, capi.ROW_MAJOR, capi.ROW_MAJOR)
+            rl = timed(capi.F16F16F16, 4095, 4097, 1023, capi.ROW_MAJOR, capi.ROW_MAJOR, 50, 50, vendor=lt)
+            extras["hipblaslt_f16_4095x4097x1023_row_row"] = {
+                "tflops": round(2.0 * 4095 * 4097 * 1023 / (rl["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                "kernel_us_mean": round(rl["kernel_ms_mean"] * 1e3, 2)}
+            lt.close()
             for name, (ty, sz, st, wu, lb, sb) in {
                     "hipblaslt_bf16_4096": (capi.BF16BF16F32, 4096, args.steps, args.warmup, capi.COL_MAJOR, 1.0),
                     "hipblaslt_s8_8192": (capi.S8S8S32, 8192, 30, 40, capi.COL_MAJOR, 1.0),

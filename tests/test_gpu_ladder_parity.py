@@ -78,6 +78,27 @@ def test_mfma_every_variant_bit_exact(G, types):
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 1, 1)), (types, variant, la, lb, m, n, k)
 
 
+@pytest.mark.parametrize("types", ALL_TYPES)
+def test_a_few_columns_past_a_tile_multiple(G, types):
+    """N one, seven or thirty-two columns past a multiple of the tile width (the last tile column is almost empty),
+    and N below 32 altogether: every variant, every layout, whole and ragged M and K; bit-exact on integer-valued
+    data, within tolerance on N(0,1) data."""
+    nvar = G.capi.variant_count(types, G.capi.RUNG_MFMA)
+    shapes = [(256, 257, 128), (300, 288, 200), (512, 513, 1024), (130, 160, 95), (257, 7, 333), (64, 32, 64)]
+    for variant, (la, lb), (m, n, k) in itertools.product(range(0, nvar + 1), LAYOUTS, shapes):
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=variant + n)
+        print("case", types, variant, la, lb, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1, 1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 1, 1)), (types, variant, la, lb, m, n, k)
+    if types == O.S8S8S32:
+        return
+    for (la, lb), (m, n, k) in itertools.product(LAYOUTS, [(512, 513, 1024), (300, 288, 1000)]):
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_NORMAL, seed=23)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 1.0, 0.5, MFMA)
+        truth, _ = O.gemm_f64(types, a, b, c, m, n, k, la, lb, 1.0, 0.5)
+        G.assert_within(types, got, truth, f"types {types} layouts {la}{lb} {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("types", SKINNY_TYPES)
 def test_skinny_rung(G, types):
     # three kernels: M <= 16 with K % 128 == 0 (direct-to-LDS), M <= 16 otherwise (registers), 16 < M <= 128 (tile)
