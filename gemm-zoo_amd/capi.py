@@ -55,6 +55,7 @@ class Plan(C.Structure):
         ("grid", C.c_int64), ("split_k", C.c_int32),
         ("vector_bytes_a", C.c_int32), ("vector_bytes_b", C.c_int32),
         ("tail_rows", C.c_int32), ("tail_tile_m", C.c_int32), ("tail_tile_n", C.c_int32), ("tail_grid", C.c_int64),
+        ("tail_cols", C.c_int32),
     ]
 
     def as_dict(self):

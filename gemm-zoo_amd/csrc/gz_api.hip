@@ -92,6 +92,7 @@ static int run(const void* A, const void* B, const void* C, void* D, int64_t M, 
   g.layoutA = layoutA; g.layoutB = layoutB;
   g.alpha = alpha; g.beta = beta;
   g.store_hint = 0;
+  g.ldb = g.ldd = (int)N;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   int resolved = resolve_rung(TYPES, M, N, K, layoutA, layoutB, rung);
@@ -282,7 +283,8 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       }
       MfmaCfg c;
       MfmaSplit sp;
-      int m_first = m;
+      MfmaColSplit cs;
+      int m_first = m, n_first = n;
       if (variant == 0 && k > 0 && mfma_resolve_split(types, m, n, k, layoutA, layoutB, num_cus, &sp)) {
         c = sp.main;
         m_first = sp.rows_main;
@@ -290,6 +292,13 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
         plan->tail_tile_m = sp.tail.bm;
         plan->tail_tile_n = sp.tail.bn;
         plan->tail_grid = (int64_t)ceil_div(m - sp.rows_main, sp.tail.bm) * ceil_div(n, sp.tail.bn);
+      } else if (variant == 0 && k > 0 && mfma_resolve_colsplit(types, m, n, k, layoutA, layoutB, num_cus, &cs)) {
+        c = cs.main;
+        n_first = cs.cols_main;
+        plan->tail_cols = n - cs.cols_main;
+        plan->tail_tile_m = cs.tail.bm;
+        plan->tail_tile_n = cs.tail.bn;
+        plan->tail_grid = (int64_t)ceil_div(m, cs.tail.bm) * ceil_div(n - cs.cols_main, cs.tail.bn);
       } else if (!mfma_resolve(types, m, n, k, layoutA, layoutB, variant, num_cus, &c)) {
         set_error("mfma rung: unknown variant %d", variant);
         return GZ_ERR_UNSUPPORTED;
@@ -299,7 +308,7 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       plan->wave_m = c.bm / c.waves_m; plan->wave_n = c.bn / c.waves_n;
       plan->threads = c.waves_m * c.waves_n * 64;
       plan->lds_bytes = mfma_lds_bytes(c);
-      plan->grid = (int64_t)ceil_div(m_first, c.bm) * ceil_div(n, c.bn);
+      plan->grid = (int64_t)ceil_div(m_first, c.bm) * ceil_div(n_first, c.bn);
       if (plan->lds_bytes > lds_per_cu) {
         set_error("mfma variant %d needs %d bytes of LDS, device has %d", c.id, plan->lds_bytes, lds_per_cu);
         return GZ_ERR_UNSUPPORTED;

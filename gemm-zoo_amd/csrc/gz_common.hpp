@@ -92,6 +92,10 @@ template <int TYPES> struct GemmArgs {
   int layoutA, layoutB;
   typename T::scalar_t alpha, beta;
   int store_hint;   // MFMA rung: 1 = the stores of D carry the non-temporal hint (set by the launcher)
+  // Row pitch in elements of a row-major B (ldb) and of C and D (ldd).  Both are N for every caller of the library;
+  // the MFMA launcher sets them apart from N when it runs a range of columns as a launch of its own, and only the
+  // kernels it then picks (register-staged tile kernel, 256x256 hand-scheduled kernel with K-contiguous B) read them.
+  int ldb, ldd;
 };
 
 // ---------------------------------------------------------------------------

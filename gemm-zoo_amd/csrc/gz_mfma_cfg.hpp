@@ -176,6 +176,46 @@ inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int 
   return true;
 }
 
+// A few columns past a multiple of 256.  N = 4097 puts one column of data into a seventeenth column of 256-wide
+// tiles, each of which costs what a whole tile costs, and where the whole ones just fill the compute units that is
+// a round of its own (fp16 4096 x 4097 x 1024, K-contiguous B: 80 us against 42 for N = 4096).  Cut off instead:
+// the first launch covers the columns up to the multiple of 256, the second the few that remain, as an M x r
+// problem on small tiles (about 0.45 of a round of whole tiles: 15-18 us at K = 1024, 44-52 at K = 4096).  Both
+// address C, D and a row-major B with the row pitch of the whole matrices (ldb / ldd of the kernel arguments), which
+// the register-staged tile kernel and the epilogues take; with a K-contiguous B the first launch keeps the
+// hand-scheduled kernel.  Taken when the estimate is at least 3 % below the single launch.
+struct MfmaColSplit {
+  int cols_main;      // columns of the first launch (a multiple of 256), 0 = no split
+  MfmaCfg main, tail;
+};
+inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaColSplit* out) {
+  out->cols_main = 0;
+  if (num_cus <= 0) num_cus = 256;
+  const int r = N % 256;
+  if (N < 512 || r == 0 || r > 64 || M <= 0 || K <= 0) return false;
+  MfmaCfg single;
+  const double cost_single = mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, &single);
+  const int cols_main = N - r;
+  MfmaCfg main_cfg, tail_cfg;
+  double cost_main = mfma_choose(types, M, cols_main, K, layoutA, layoutB, num_cus, &main_cfg);
+  // the first launch keeps a direct-to-LDS kernel only with row-major A, K-contiguous B and a 256 x 256 tile
+  const int cls = mfma_shape_class(main_cfg, mfma_in_size(types), M, cols_main, K, layoutA, layoutB);
+  const bool direct_before = layoutA == GZ_ROW_MAJOR && types != GZ_F32F32F32 &&
+                             (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && main_cfg.bm == 256 && main_cfg.bn == 256));
+  const bool direct_after = direct_before && layoutB == GZ_COL_MAJOR && main_cfg.bm == 256 && main_cfg.bn == 256;
+  if (direct_before && !direct_after) cost_main *= 2.2;
+  // on the register-staged kernel eight waves carry a 256 x 256 tile of 16-bit elements better than four
+  // (fp16 4095 x 4097 x 1023, row-major B: 119 us against 158)
+  if (!direct_after && main_cfg.bm == 256 && main_cfg.bn == 256 && mfma_in_size(types) == 2) main_cfg = kMfmaCfgs[6];
+  tail_cfg = kMfmaCfgs[2];   // 128 x 128: the strip in as many work-groups as it has row blocks
+  const double cost_tail = 0.45 * ((M + 4095) / 4096);
+  if (cost_main + cost_tail > 0.97 * cost_single) return false;
+  out->cols_main = cols_main;
+  out->main = main_cfg;
+  out->tail = tail_cfg;
+  return true;
+}
+
 // Shape class of a launch: the direct-to-LDS kernels also need 16-byte aligned operands.
 inline int mfma_launch_class(const MfmaCfg& c, int in_size, int M, int N, int K, int layoutA, int layoutB, const void* A,
                              const void* B, const void* C, const void* D) {

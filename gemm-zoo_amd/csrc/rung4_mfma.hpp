@@ -102,7 +102,7 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
 template <int TYPES, int FM, int FN, class Acc>
 __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc (&acc)[FM][FN], int row0, int col0, int lane) {
   using out_t = typename Traits<TYPES>::out_t;
-  const int N = g.N;
+  const int LDD = g.ldd;
   const bool use_c = g.beta != 0;
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
@@ -112,7 +112,7 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
       static_for<4>([&](auto q_c) {
         constexpr int Q = decltype(q_c)::value;
         const int n = col0 + 32 * J + 8 * Q + 4 * (lane >> 5);
-        const size_t o = (size_t)m * N + n;
+        const size_t o = (size_t)m * LDD + n;
         const Acc& a = acc[I][J];
         out_t cv[4] = {0, 0, 0, 0}, dv[4];
         if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
@@ -142,7 +142,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   using acc_t = typename Traits<TYPES>::acc_t;
   constexpr int COLS = FN * 32, PITCH_E = COLS * 4 + 16;
   constexpr int LPR = COLS / 4, RPI = 64 / LPR, NI = 32 / RPI;   // lanes per row, rows per instruction, instructions
-  const int M = g.M, N = g.N;
+  const int M = g.M, N = g.N, LDD = g.ldd;   // LDD: elements between the rows of C and D (N unless the launch covers a column range)
   const bool use_c = g.beta != 0;
   char* wr = region + (lane & 31) * PITCH_E + (lane >> 5) * 16;
   const char* rd = region + (lane / LPR) * PITCH_E + (lane % LPR) * 16;
@@ -152,7 +152,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   // otherwise the block is written one element per lane with the lanes along a row, which is still whole cache
   // lines per instruction (fp16 4095 x 4097 x 63 took 65 us with four scattered 2-byte stores per lane).
   constexpr uintptr_t VEC_ALIGN = 4 * sizeof(out_t) - 1;
-  const bool vec = !RAGGED || ((N & 3) == 0 && ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & VEC_ALIGN) == 0);
+  const bool vec = !RAGGED || ((N & 3) == 0 && (LDD & 3) == 0 && ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & VEC_ALIGN) == 0);
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
     // the block's values of C first: their latency passes while the accumulators go through LDS
@@ -161,7 +161,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       constexpr int T = decltype(t_c)::value;
       cv[T][0] = cv[T][1] = cv[T][2] = cv[T][3] = 0;
       const int m = row0 + 32 * I + T * RPI + lane / LPR;
-      if (use_c && vec && (!RAGGED || (m < M && n < N))) __builtin_memcpy(cv[T], g.C + (size_t)m * N + n, sizeof(cv[T]));
+      if (use_c && vec && (!RAGGED || (m < M && n < N))) __builtin_memcpy(cv[T], g.C + (size_t)m * LDD + n, sizeof(cv[T]));
     });
     static_for<FN>([&](auto j_c) {
       constexpr int J = decltype(j_c)::value;
@@ -180,7 +180,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         acc_t v[4];
         __builtin_memcpy(v, rd + T * RPI * PITCH_E, 16);
         const int m = row0 + 32 * I + T * RPI + lane / LPR;
-        const size_t o = (size_t)m * N + n;
+        const size_t o = (size_t)m * LDD + n;
         if constexpr (RAGGED) {
           if (m >= M || n >= N) return;   // N is a multiple of four here: the lane's four columns end together
         }
@@ -212,7 +212,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
           const int nn = col0 + c0 + lane;
           acc_t v;
           __builtin_memcpy(&v, region + r * PITCH_E + (c0 + lane) * 4, 4);
-          const size_t o = (size_t)m * N + nn;
+          const size_t o = (size_t)m * LDD + nn;
           if (nn < N) g.D[o] = epilogue<TYPES>(v, g.alpha, g.beta, g.C + o);
         }
       }
@@ -243,17 +243,17 @@ constexpr int PITCH = SLAB_BYTES + 16;    // LDS row pitch
 constexpr int KSTEPS = SLAB_BYTES / 32;   // MFMA steps per slab
 
 // 16-byte global load of `EPV` elements starting at element (line, pos) of a
-// matrix whose lines are `extent` long.  With EDGE the access is predicated and
+// matrix whose lines are `extent` long and `pitch` elements apart.  With EDGE the access is predicated and
 // zero-filled, and may be unaligned (gfx950 global loads tolerate that).
 template <typename in_t, bool EDGE>
-__device__ inline u32x4_t load16(const in_t* __restrict__ base, int line, int lines, int pos, int extent) {
+__device__ inline u32x4_t load16(const in_t* __restrict__ base, int line, int lines, int pos, int extent, int pitch) {
   constexpr int EPV = 16 / (int)sizeof(in_t);
   if constexpr (!EDGE) {
-    return *reinterpret_cast<const u32x4_t*>(base + (size_t)line * extent + pos);
+    return *reinterpret_cast<const u32x4_t*>(base + (size_t)line * pitch + pos);
   } else {
     u32x4_t v = {0u, 0u, 0u, 0u};
     if (line < lines) {
-      const in_t* p = base + (size_t)line * extent + pos;
+      const in_t* p = base + (size_t)line * pitch + pos;
       if (pos + EPV <= extent) {
         __builtin_memcpy(&v, p, 16);
       } else if (pos < extent) {
@@ -344,14 +344,15 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
   // bytes of one staged slab of this operand
   static constexpr int LDS_BYTES = (!KC && ES == 4) ? BK * NAT_PITCH : ROWS * PITCH;
 
-  // rows_total: M or N ; row0: first tile row ; k0: first k of the slab
-  __device__ inline void load(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid) {
+  // rows_total: M or N ; row0: first tile row ; k0: first k of the slab ; pitch: elements between the k lines of an
+  // operand whose lines run along M / N (rows_total unless the launch covers a range of columns of a wider matrix)
+  __device__ inline void load(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid, int pitch) {
     if constexpr (KC) {
 #pragma unroll
       for (int it = 0; it < VECS; it++) {
         const int id = it * NT + tid;
         const int row = id >> 3, c = id & 7;
-        r[it] = load16<in_t, EDGE>(base, row0 + row, rows_total, k0 + c * EPV, K);
+        r[it] = load16<in_t, EDGE>(base, row0 + row, rows_total, k0 + c * EPV, K, K);
       }
     } else {
 #pragma unroll
@@ -360,7 +361,7 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
         unit_of(u * NT + tid, mc, ku);
 #pragma unroll
         for (int t = 0; t < TR; t++)
-          r[u * TR + t] = load16<in_t, EDGE>(base, k0 + ku * TR + t, K, row0 + mc * EPV, rows_total);
+          r[u * TR + t] = load16<in_t, EDGE>(base, k0 + ku * TR + t, K, row0 + mc * EPV, rows_total, pitch);
       }
     }
   }
@@ -521,13 +522,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   };
 
   // Prologue: slab 0 into LDS, slab 1 parked in registers, fragments of (slab 0, step 0) requested.
-  sa.load(g.A, g.M, g.K, m0, 0, tid);
-  sb.load(g.B, g.N, g.K, n0, 0, tid);
+  sa.load(g.A, g.M, g.K, m0, 0, tid, g.M);
+  sb.load(g.B, g.N, g.K, n0, 0, tid, g.ldb);
   sa.store(lds, tid);
   sb.store(lds + A_BYTES, tid);
   if (ktiles > 1) {
-    sa.load(g.A, g.M, g.K, m0, BK, tid);
-    sb.load(g.B, g.N, g.K, n0, BK, tid);
+    sa.load(g.A, g.M, g.K, m0, BK, tid, g.M);
+    sb.load(g.B, g.N, g.K, n0, BK, tid, g.ldb);
   }
   __syncthreads();
   read_frags(0, lds, 0);
@@ -563,8 +564,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       sa.store(nxt, tid);
       sb.store(nxt + A_BYTES, tid);
       const int k_next = (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK;
-      sa.load(g.A, g.M, g.K, m0, k_next, tid);
-      sb.load(g.B, g.N, g.K, n0, k_next, tid);
+      sa.load(g.A, g.M, g.K, m0, k_next, tid, g.M);
+      sb.load(g.B, g.N, g.K, n0, k_next, tid, g.ldb);
       mma2(0);
       mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, FM * FN>();
       __builtin_amdgcn_sched_barrier(0);
@@ -584,8 +585,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     sa.store(nxt, tid);
     sb.store(nxt + A_BYTES, tid);
     const int k_next = (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK;
-    sa.load(g.A, g.M, g.K, m0, k_next, tid);
-    sb.load(g.B, g.N, g.K, n0, k_next, tid);
+    sa.load(g.A, g.M, g.K, m0, k_next, tid, g.M);
+    sb.load(g.B, g.N, g.K, n0, k_next, tid, g.ldb);
     mma(0);
     mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, MFMAS_PER_STEP>();
     __builtin_amdgcn_sched_barrier(0);
@@ -1209,7 +1210,11 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
 
 template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& cfg, hipStream_t s) {
   using in_t = typename Traits<TYPES>::in_t;
-  const int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
+  int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
+  // a column range of wider matrices: only the register-staged kernel reads the pitch of a row-major B, and the
+  // epilogue that reads the pitch of C and D unaligned is the one of the ragged kernels
+  if (g.layoutB == GZ_ROW_MAJOR && g.ldb != g.N) edge = MFMA_SHAPE_GENERAL;
+  else if (g.ldd != g.N && edge == MFMA_SHAPE_WHOLE) edge = MFMA_SHAPE_RAGGED_MN;
   switch (cfg.id) {
     case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
     case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);
@@ -1240,6 +1245,21 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       const int st = launch_one<TYPES>(top, sp.main, s);
       if (st != GZ_OK) return st;
       return launch_one<TYPES>(bottom, sp.tail, s);
+    }
+  }
+  if (variant == 0 && g.K > 0) {
+    // a few columns past a multiple of 256: those columns in a launch of their own
+    MfmaColSplit cs;
+    if (mfma_resolve_colsplit(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, 256, &cs)) {
+      GemmArgs<TYPES> left = g, right = g;
+      left.N = cs.cols_main;
+      right.N = g.N - cs.cols_main;
+      right.B = g.layoutB == GZ_ROW_MAJOR ? g.B + cs.cols_main : g.B + (size_t)cs.cols_main * g.K;
+      if (g.C) right.C = g.C + cs.cols_main;
+      right.D = g.D + cs.cols_main;
+      const int st = launch_one<TYPES>(left, cs.main, s);
+      if (st != GZ_OK) return st;
+      return launch_one<TYPES>(right, cs.tail, s);
     }
   }
   MfmaCfg cfg;

@@ -120,6 +120,10 @@ typedef struct gz_plan_t {
   int32_t tail_rows;
   int32_t tail_tile_m, tail_tile_n;
   int64_t tail_grid;
+  /* The same for columns: N a few columns past a multiple of 256 would put them into a tile column of their own
+   * that costs as much as a whole one; the last tail_cols columns then run in a second launch (tail_tile_*,
+   * tail_grid describe it; 0: no such split; never together with tail_rows).                                  */
+  int32_t tail_cols;
 } gz_plan_t;
 
 /* variant: 0 = launcher's choice; other values select a tile configuration of the rung

@@ -152,7 +152,7 @@ def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile):
 
 def test_ragged_grid_takes_the_small_tile(G):
     # N = 4097 would need a 17th column of 256-wide tiles for one column of data
-    assert G.capi.plan(O.F16F16F16, 4095, 4097, 1023, O.ROW, O.ROW).tile_m == 128
+    assert G.capi.plan(O.F16F16F16, 4095, 4096 + 100, 1023, O.ROW, O.ROW).tile_m == 128
     assert G.capi.plan(O.BF16BF16F32, 4096, 4096, 4096, O.ROW, O.COL).tile_m == 256
     assert G.capi.plan(O.BF16BF16F32, 2048, 2048, 2048, O.ROW, O.COL).tile_m == 128
 
@@ -207,3 +207,35 @@ def test_mostly_empty_last_round_runs_as_two_launches(G, types, shape, lb):
     got0 = G.run_gemm(types, ha, hb, None, m, n, k, O.ROW, lb, 1, 0, -1)
     ref = O.gemm(types, ha, hb, None, m, n, k, O.ROW, lb, 1, 0, rows=(seam - 4, seam + 4))
     assert np.array_equal(got0[seam - 4:seam + 4], ref[seam - 4:seam + 4])
+
+
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32, O.E4M3E4M3F16])
+@pytest.mark.parametrize("shape", [(4096, 4097, 72), (2048, 8200, 130), (4095, 4160, 255)])
+def test_columns_past_a_multiple_of_256_run_as_a_second_launch(G, types, shape):
+    """N = 256 q + r with r <= 64 on a grid that the whole tiles just fill: the launcher's choice gives the last r
+    columns a launch of their own, which addresses C, D and a row-major B with the pitch of the whole matrices.
+    Every layout, alpha and beta at work, whole and ragged K; bit-exact on integer-valued data against the oracle
+    (first and last rows, every column)."""
+    m, n, k = shape
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+    split_seen = False
+    for la, lb in [(O.ROW, O.COL), (O.ROW, O.ROW), (O.COL, O.ROW), (O.COL, O.COL)]:
+        p = G.capi.plan(types, m, n, k, la, lb)
+        split_seen |= p.tail_cols > 0
+        if p.tail_cols:
+            assert p.tail_cols == n % 256 and p.tail_rows == 0 and (p.tail_tile_m, p.tail_tile_n) == (128, 128)
+            assert p.grid == -(-m // p.tile_m) * ((n - p.tail_cols) // p.tile_n)
+        a, b, c = O.make_inputs(types, m, n, k, kind=kind, seed=5 + la + 2 * lb)
+        print("case", types, shape, la, lb, p.tail_cols, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, 2, -1, -1)
+        for rows in ((0, 24), (m - 24, m)):
+            ref = O.gemm(types, a, b, c, m, n, k, la, lb, 2, -1, rows=rows)
+            assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, shape, la, lb, rows)
+    assert split_seen
+
+
+def test_ragged_baseline_shape_is_split_by_columns(G):
+    p = G.capi.plan(O.F16F16F16, 4095, 4097, 1023, O.ROW, O.ROW)
+    assert (p.tile_m, p.tile_n, p.grid, p.tail_cols, p.tail_grid) == (256, 256, 256, 1, 32)
+    assert G.capi.plan(O.F16F16F16, 4096, 4096, 1024, O.ROW, O.ROW).tail_cols == 0
+    assert G.capi.plan(O.F16F16F16, 4096, 4096 + 100, 1024, O.ROW, O.ROW).tail_cols == 0
