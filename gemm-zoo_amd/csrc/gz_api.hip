@@ -296,9 +296,15 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
         c = cs.main;
         n_first = cs.cols_main;
         plan->tail_cols = n - cs.cols_main;
-        plan->tail_tile_m = cs.tail.bm;
-        plan->tail_tile_n = cs.tail.bn;
-        plan->tail_grid = (int64_t)ceil_div(m, cs.tail.bm) * ceil_div(n - cs.cols_main, cs.tail.bn);
+        if (plan->tail_cols <= MFMA_STRIP_MAX_COLS) {   // dot products, one wave per row, four rows per work-group
+          plan->tail_tile_m = 4;
+          plan->tail_tile_n = plan->tail_cols;
+          plan->tail_grid = ceil_div(m, 4);
+        } else {
+          plan->tail_tile_m = cs.tail.bm;
+          plan->tail_tile_n = cs.tail.bn;
+          plan->tail_grid = (int64_t)ceil_div(m, cs.tail.bm) * ceil_div(n - cs.cols_main, cs.tail.bn);
+        }
       } else if (!mfma_resolve(types, m, n, k, layoutA, layoutB, variant, num_cus, &c)) {
         set_error("mfma rung: unknown variant %d", variant);
         return GZ_ERR_UNSUPPORTED;

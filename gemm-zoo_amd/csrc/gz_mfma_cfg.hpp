@@ -179,11 +179,13 @@ inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int 
 // A few columns past a multiple of 256.  N = 4097 puts one column of data into a seventeenth column of 256-wide
 // tiles, each of which costs what a whole tile costs, and where the whole ones just fill the compute units that is
 // a round of its own (fp16 4096 x 4097 x 1024, K-contiguous B: 80 us against 42 for N = 4096).  Cut off instead:
-// the first launch covers the columns up to the multiple of 256, the second the few that remain, as an M x r
-// problem on small tiles (about 0.45 of a round of whole tiles: 15-18 us at K = 1024, 44-52 at K = 4096).  Both
+// the first launch covers the columns up to the multiple of 256, the second the few that remain: up to
+// MFMA_STRIP_MAX_COLS of them as dot products, one wave per row (mfma_strip_kernel), more as an M x r problem on small
+// tiles (about 0.45 of a round of whole tiles: 15-18 us at K = 1024, 44-52 at K = 4096).  Both
 // address C, D and a row-major B with the row pitch of the whole matrices (ldb / ldd of the kernel arguments), which
 // the register-staged tile kernel and the epilogues take; with a K-contiguous B the first launch keeps the
 // hand-scheduled kernel.  Taken when the estimate is at least 3 % below the single launch.
+constexpr int MFMA_STRIP_MAX_COLS = 8;   // up to here the cut-off columns run as dot products (mfma_strip_kernel), not as tiles
 struct MfmaColSplit {
   int cols_main;      // columns of the first launch (a multiple of 256), 0 = no split
   MfmaCfg main, tail;
@@ -208,7 +210,7 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   // (fp16 4095 x 4097 x 1023, row-major B: 119 us against 158)
   if (!direct_after && main_cfg.bm == 256 && main_cfg.bn == 256 && mfma_in_size(types) == 2) main_cfg = kMfmaCfgs[6];
   tail_cfg = kMfmaCfgs[2];   // 128 x 128: the strip in as many work-groups as it has row blocks
-  const double cost_tail = 0.45 * ((M + 4095) / 4096);
+  const double cost_tail = (r <= MFMA_STRIP_MAX_COLS ? 0.15 : 0.45) * ((M + 4095) / 4096);
   if (cost_main + cost_tail > 0.97 * cost_single) return false;
   out->cols_main = cols_main;
   out->main = main_cfg;

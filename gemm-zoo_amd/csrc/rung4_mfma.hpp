@@ -1208,6 +1208,97 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   return GZ_OK;
 }
 
+// ---------------------------------------------------------------------------
+// The last few columns of a problem whose N is just past a multiple of 256 (see mfma_resolve_colsplit), at most
+// STRIP_MAX_COLS of them: g.N columns, g.B / g.C / g.D pointing at the first of them, ldb / ldd the pitch of the
+// whole matrices.  As a tile problem this strip is all edge (fp16 4095 x 1 x 1023 took 47 us on 128 x 128 tiles, most
+// of it element-wise loads of one column of B); as M dot products per column it is one pass over A.  One wave per
+// row: the lanes take 16-byte pieces of the row (and of the columns of a K-contiguous B; a row-major B is gathered),
+// multiply-add on the vector ALUs in the accumulator type, and meet in a butterfly over the 64 lanes.
+// ---------------------------------------------------------------------------
+constexpr int STRIP_ROWS_PER_WG = 4;
+template <int TYPES, bool A_KC, bool B_KC, int R>
+__global__ void __launch_bounds__(STRIP_ROWS_PER_WG * 64) mfma_strip_kernel(GemmArgs<TYPES> g) {
+  using T = Traits<TYPES>;
+  using in_t = typename T::in_t;
+  using acc_t = typename T::acc_t;
+  constexpr int EPV = 16 / (int)sizeof(in_t);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int m = blockIdx.x * STRIP_ROWS_PER_WG + wave;
+  if (m >= g.M) return;
+  const int K = g.K, M = g.M, r = g.N, ldb = g.ldb;
+  acc_t acc[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) acc[j] = 0;
+  auto mac = [&](acc_t a, acc_t b, acc_t c) -> acc_t {
+    if constexpr (T::is_int) return c + a * b;
+    else return __builtin_fmaf(a, b, c);
+  };
+  const int kv = K / EPV;   // whole 16-byte pieces of a K line
+  for (int v = lane; v < kv; v += 64) {
+    const int k0 = v * EPV;
+    in_t a[EPV];
+    if constexpr (A_KC) {
+      __builtin_memcpy(a, g.A + (size_t)m * K + k0, 16);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; e++) a[e] = g.A[(size_t)(k0 + e) * M + m];
+    }
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      if (j < r) {   // the same for every lane
+        in_t b[EPV];
+        if constexpr (B_KC) {
+          __builtin_memcpy(b, g.B + (size_t)j * K + k0, 16);
+        } else {
+#pragma unroll
+          for (int e = 0; e < EPV; e++) b[e] = g.B[(size_t)(k0 + e) * ldb + j];
+        }
+#pragma unroll
+        for (int e = 0; e < EPV; e++) acc[j] = mac(widen_in<TYPES>(a[e]), widen_in<TYPES>(b[e]), acc[j]);
+      }
+    }
+  }
+  const int k = kv * EPV + lane;   // what is left of a ragged K, one element per lane
+  if (k < K) {
+    const acc_t a = widen_in<TYPES>(A_KC ? g.A[(size_t)m * K + k] : g.A[(size_t)k * M + m]);
+#pragma unroll
+    for (int j = 0; j < R; j++)
+      if (j < r) acc[j] = mac(a, widen_in<TYPES>(B_KC ? g.B[(size_t)j * K + k] : g.B[(size_t)k * ldb + j]), acc[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < R; j++)
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) acc[j] += __shfl_xor(acc[j], off, 64);
+  if (lane == 0) {
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      if (j < r) {
+        const size_t o = (size_t)m * g.ldd + j;
+        g.D[o] = epilogue<TYPES>(acc[j], g.alpha, g.beta, g.C + o);
+      }
+    }
+  }
+}
+
+template <int TYPES> static int launch_strip(const GemmArgs<TYPES>& g, hipStream_t s) {
+  const dim3 grid((unsigned)ceil_div(g.M, STRIP_ROWS_PER_WG)), block(STRIP_ROWS_PER_WG * 64);
+  const bool akc = g.layoutA == GZ_ROW_MAJOR, bkc = g.layoutB == GZ_COL_MAJOR;
+#define GZ_STRIP(AKC, BKC)                                                                              \
+  do {                                                                                                  \
+    if (g.N <= 1) hipLaunchKernelGGL((mfma_strip_kernel<TYPES, AKC, BKC, 1>), grid, block, 0, s, g);     \
+    else if (g.N <= 4) hipLaunchKernelGGL((mfma_strip_kernel<TYPES, AKC, BKC, 4>), grid, block, 0, s, g); \
+    else hipLaunchKernelGGL((mfma_strip_kernel<TYPES, AKC, BKC, MFMA_STRIP_MAX_COLS>), grid, block, 0, s, g); \
+  } while (0)
+  if (akc && bkc) GZ_STRIP(true, true);
+  else if (akc) GZ_STRIP(true, false);
+  else if (bkc) GZ_STRIP(false, true);
+  else GZ_STRIP(false, false);
+#undef GZ_STRIP
+  GZ_HIP_TRY(hipGetLastError());
+  return GZ_OK;
+}
+
 template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& cfg, hipStream_t s) {
   using in_t = typename Traits<TYPES>::in_t;
   int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
@@ -1259,7 +1350,7 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       right.D = g.D + cs.cols_main;
       const int st = launch_one<TYPES>(left, cs.main, s);
       if (st != GZ_OK) return st;
-      return launch_one<TYPES>(right, cs.tail, s);
+      return right.N <= MFMA_STRIP_MAX_COLS ? launch_strip<TYPES>(right, s) : launch_one<TYPES>(right, cs.tail, s);
     }
   }
   MfmaCfg cfg;
