@@ -109,7 +109,10 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
     const bool direct = a_rows && types != GZ_F32F32F32 &&
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
-    const double shape_cost = i == 0 ? (double)rounds : i == 1 ? 0.75 * rounds : 0.40 + 0.27 * rounds;
+    // (128 x 128 beyond four rounds: each further round costs a little more, 6144^2 x 6144 = 9 rounds measured
+    // 478 us against 457 for three rounds of 256 x 256)
+    const double shape_cost = i == 0 ? (double)rounds : i == 1 ? 0.75 * rounds
+                                     : 0.40 + 0.27 * rounds + 0.035 * (rounds > 4 ? rounds - 4 : 0);
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
     const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : 1.15) : 1.0;
     const double cost = shape_cost * rowb * (direct ? 1.0 : 2.2);
