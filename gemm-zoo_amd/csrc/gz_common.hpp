@@ -91,7 +91,7 @@ template <int TYPES> struct GemmArgs {
   int M, N, K;
   int layoutA, layoutB;
   typename T::scalar_t alpha, beta;
-  int store_hint;   // MFMA rung: 1 = the stores of D carry the non-temporal hint (set by the launcher)
+  int store_hint;   // MFMA rung, set by the launcher: bit 0 = the stores of D carry the non-temporal hint, bit 1 = the loads of C
   // Row pitch in elements of a row-major B (ldb) and of C and D (ldd).  Both are N for every caller of the library;
   // the MFMA launcher sets them apart from N when it runs a range of columns as a launch of its own, and only the
   // kernels it then picks (register-staged tile kernel, 256x256 hand-scheduled kernel with K-contiguous B) read them.

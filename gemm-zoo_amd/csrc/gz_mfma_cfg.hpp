@@ -85,11 +85,13 @@ inline int mfma_in_size(int types) {
 // mostly the writing of an output larger than that loses with the hint (int8 8192 x 8192 x {128, 512, 1024, 2048}
 // 65 / 77, 86 / 96, 106 / 115, 158 / 163; bf16 8192 x 8192 x 256 80 / 88): the last-level cache no longer takes the
 // burst in.  In between (6144^2 x 4096, int8 8192^2 x 4096) it makes no difference.
+// Bit 1: the loads of C (beta != 0) carry the hint as well.  That helps only in the many-rounds case (bf16 8192^3 with
+// alpha = beta = 1: 940 / 927 us, int8 561 / 548) and costs on a 64 MiB output (bf16 4096^3: 128.7 / 132.1).
 inline int mfma_store_hint(int types, long long M, long long N, long long K, int out_size, int num_cus) {
-  const long long out_bytes = M * N * out_size;
-  if (out_bytes <= (64ll << 20)) return 1;
   const long long tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  return (tiles >= 4ll * num_cus && K * mfma_in_size(types) >= 8192) ? 1 : 0;
+  if (tiles >= 4ll * num_cus && K * mfma_in_size(types) >= 8192) return 3;
+  const long long out_bytes = M * N * out_size;
+  return out_bytes <= (64ll << 20) ? 1 : 0;
 }
 
 // The launcher's own choice for one launch over the whole problem; returns the estimate it was chosen by.

@@ -161,7 +161,19 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       constexpr int T = decltype(t_c)::value;
       cv[T][0] = cv[T][1] = cv[T][2] = cv[T][3] = 0;
       const int m = row0 + 32 * I + T * RPI + lane / LPR;
-      if (use_c && vec && (!RAGGED || (m < M && n < N))) __builtin_memcpy(cv[T], g.C + (size_t)m * LDD + n, sizeof(cv[T]));
+      if (use_c && vec && (!RAGGED || (m < M && n < N))) {
+        if (g.store_hint & 2) {   // non-temporal: see mfma_store_hint
+          if constexpr (sizeof(out_t) == 4) {
+            const u32x4_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.C + (size_t)m * LDD + n));
+            __builtin_memcpy(cv[T], &w, 16);
+          } else {
+            const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(g.C + (size_t)m * LDD + n));
+            __builtin_memcpy(cv[T], &w, 8);
+          }
+        } else {
+          __builtin_memcpy(cv[T], g.C + (size_t)m * LDD + n, sizeof(cv[T]));
+        }
+      }
     });
     static_for<FN>([&](auto j_c) {
       constexpr int J = decltype(j_c)::value;
@@ -189,7 +201,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         dv[1] = epilogue<TYPES>(v[1], g.alpha, g.beta, &cv[T][1]);
         dv[2] = epilogue<TYPES>(v[2], g.alpha, g.beta, &cv[T][2]);
         dv[3] = epilogue<TYPES>(v[3], g.alpha, g.beta, &cv[T][3]);
-        if (g.store_hint) {   // non-temporal: see mfma_store_hint
+        if (g.store_hint & 1) {   // non-temporal: see mfma_store_hint
           if constexpr (sizeof(out_t) == 4) {
             u32x4_t w;
             __builtin_memcpy(&w, dv, 16);
