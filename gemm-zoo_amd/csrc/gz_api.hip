@@ -309,6 +309,11 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
         set_error("mfma rung: unknown variant %d", variant);
         return GZ_ERR_UNSUPPORTED;
       }
+      if (variant == 0) {   // as the launcher does, with 16-byte aligned operands assumed
+        int cls = mfma_shape_class(c, es, m_first, n_first, k, layoutA, layoutB);
+        if (plan->tail_cols && layoutB == GZ_ROW_MAJOR) cls = MFMA_SHAPE_GENERAL;
+        mfma_adjust_general(types, cls, layoutA, &c);
+      }
       plan->variant = c.id;
       plan->tile_m = c.bm; plan->tile_n = c.bn; plan->tile_k = MFMA_SLAB_BYTES / es;
       plan->wave_m = c.bm / c.waves_m; plan->wave_n = c.bn / c.waves_n;

@@ -144,6 +144,17 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
   return true;
 }
 
+// The launcher's choice once the class of the launch is known.  A 256 x 256 tile that has to run on the register-staged
+// kernel (ragged K, unaligned operands) wants eight waves for 8-bit integers and 16-bit floats with a row-major A
+// (4096 x 4096 x 4000, us, four / eight waves: int8 96 / 82 and 103 / 84 with a row-major B, bf16 161 / 133 and
+// 180 / 149) and four for the 8-bit floats, whose eight-wave instance does not fit its registers (105 / 206).
+inline void mfma_adjust_general(int types, int cls, int layoutA, MfmaCfg* c) {
+  if (cls != MFMA_SHAPE_GENERAL || c->bm != 256 || c->bn != 256) return;
+  const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
+  if (f8) *c = kMfmaCfgs[0];
+  else if (types != GZ_F32F32F32 && layoutA == GZ_ROW_MAJOR) *c = kMfmaCfgs[1];
+}
+
 // Ragged last round.  When the 256x256 tiles of a problem fill some rounds of the compute units and then leave a
 // last round mostly empty (6144 x 6144: 576 tiles = 2.25 rounds of 256), one launch pays for a whole round more.
 // With a row-major A the rows of the problem can be cut in two launches instead, since row ranges of A, C and D

@@ -1311,13 +1311,15 @@ template <int TYPES> static int launch_strip(const GemmArgs<TYPES>& g, hipStream
   return GZ_OK;
 }
 
-template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& cfg, hipStream_t s) {
+template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& chosen, hipStream_t s, bool adjust = false) {
   using in_t = typename Traits<TYPES>::in_t;
+  MfmaCfg cfg = chosen;
   int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
   // a column range of wider matrices: only the register-staged kernel reads the pitch of a row-major B, and the
   // epilogue that reads the pitch of C and D unaligned is the one of the ragged kernels
   if (g.layoutB == GZ_ROW_MAJOR && g.ldb != g.N) edge = MFMA_SHAPE_GENERAL;
   else if (g.ldd != g.N && edge == MFMA_SHAPE_WHOLE) edge = MFMA_SHAPE_RAGGED_MN;
+  if (adjust) mfma_adjust_general(TYPES, edge, g.layoutA, &cfg);   // launcher's choice: the wave count follows the kernel
   switch (cfg.id) {
     case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
     case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);
@@ -1345,9 +1347,9 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       bottom.A = g.A + (size_t)sp.rows_main * g.K;   // row-major A: a row range is a packed matrix
       if (g.C) bottom.C = g.C + (size_t)sp.rows_main * g.N;
       bottom.D = g.D + (size_t)sp.rows_main * g.N;
-      const int st = launch_one<TYPES>(top, sp.main, s);
+      const int st = launch_one<TYPES>(top, sp.main, s, true);
       if (st != GZ_OK) return st;
-      return launch_one<TYPES>(bottom, sp.tail, s);
+      return launch_one<TYPES>(bottom, sp.tail, s, true);
     }
   }
   if (variant == 0 && g.K > 0) {
@@ -1360,9 +1362,9 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       right.B = g.layoutB == GZ_ROW_MAJOR ? g.B + cs.cols_main : g.B + (size_t)cs.cols_main * g.K;
       if (g.C) right.C = g.C + cs.cols_main;
       right.D = g.D + cs.cols_main;
-      const int st = launch_one<TYPES>(left, cs.main, s);
+      const int st = launch_one<TYPES>(left, cs.main, s, true);
       if (st != GZ_OK) return st;
-      return right.N <= MFMA_STRIP_MAX_COLS ? launch_strip<TYPES>(right, s) : launch_one<TYPES>(right, cs.tail, s);
+      return right.N <= MFMA_STRIP_MAX_COLS ? launch_strip<TYPES>(right, s) : launch_one<TYPES>(right, cs.tail, s, true);
     }
   }
   MfmaCfg cfg;
@@ -1370,7 +1372,7 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
     set_error("mfma rung: unknown variant %d", variant);
     return GZ_ERR_UNSUPPORTED;
   }
-  return launch_one<TYPES>(g, cfg, s);
+  return launch_one<TYPES>(g, cfg, s, variant == 0);
 }
 
 }  // namespace gz
