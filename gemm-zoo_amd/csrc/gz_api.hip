@@ -296,10 +296,10 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
         c = cs.main;
         n_first = cs.cols_main;
         plan->tail_cols = n - cs.cols_main;
-        if (plan->tail_cols <= MFMA_STRIP_MAX_COLS) {   // dot products, one wave per row, four rows per work-group
-          plan->tail_tile_m = 4;
+        if (plan->tail_cols <= MFMA_STRIP_MAX_COLS) {   // dot products, one wave per row, sixteen rows per work-group
+          plan->tail_tile_m = 16;
           plan->tail_tile_n = plan->tail_cols;
-          plan->tail_grid = ceil_div(m, 4);
+          plan->tail_grid = ceil_div(m, 16);
         } else {
           plan->tail_tile_m = cs.tail.bm;
           plan->tail_tile_n = cs.tail.bn;

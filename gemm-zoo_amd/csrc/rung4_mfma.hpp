@@ -1225,76 +1225,84 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
 // STRIP_MAX_COLS of them: g.N columns, g.B / g.C / g.D pointing at the first of them, ldb / ldd the pitch of the
 // whole matrices.  As a tile problem this strip is all edge (fp16 4095 x 1 x 1023 took 47 us on 128 x 128 tiles, most
 // of it element-wise loads of one column of B); as M dot products per column it is one pass over A.  One wave per
-// row: the lanes take 16-byte pieces of the row (and of the columns of a K-contiguous B; a row-major B is gathered),
-// multiply-add on the vector ALUs in the accumulator type, and meet in a butterfly over the 64 lanes.
+// row, four rows per wave: the lanes take 16-byte pieces of the row and of the columns (staged in LDS), multiply-add on
+// the vector ALUs in the accumulator type, and meet in a butterfly over the 64 lanes.
 // ---------------------------------------------------------------------------
-constexpr int STRIP_ROWS_PER_WG = 4;
+constexpr int STRIP_WAVES = 4, STRIP_ROWS_PER_WAVE = 4, STRIP_ROWS_PER_WG = STRIP_WAVES * STRIP_ROWS_PER_WAVE;
+constexpr int STRIP_K_CHUNK = 2048;   // k values of the strip's columns held in LDS at a time
 template <int TYPES, bool A_KC, bool B_KC, int R>
-__global__ void __launch_bounds__(STRIP_ROWS_PER_WG * 64) mfma_strip_kernel(GemmArgs<TYPES> g) {
+__global__ void __launch_bounds__(STRIP_WAVES * 64) mfma_strip_kernel(GemmArgs<TYPES> g) {
   using T = Traits<TYPES>;
   using in_t = typename T::in_t;
   using acc_t = typename T::acc_t;
   constexpr int EPV = 16 / (int)sizeof(in_t);
+  // The columns of B go through LDS, K-contiguous, once per work-group: gathered by every wave from a row-major B
+  // (one cache line per element) they were most of the kernel's time (19 us for one column of 1023).
+  __shared__ __attribute__((aligned(16))) in_t bs[R * STRIP_K_CHUNK];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int m = blockIdx.x * STRIP_ROWS_PER_WG + wave;
-  if (m >= g.M) return;
+  const int m0 = blockIdx.x * STRIP_ROWS_PER_WG + wave * STRIP_ROWS_PER_WAVE;
   const int K = g.K, M = g.M, r = g.N, ldb = g.ldb;
-  acc_t acc[R];
+  acc_t acc[STRIP_ROWS_PER_WAVE][R];
 #pragma unroll
-  for (int j = 0; j < R; j++) acc[j] = 0;
+  for (int i = 0; i < STRIP_ROWS_PER_WAVE; i++)
+#pragma unroll
+    for (int j = 0; j < R; j++) acc[i][j] = 0;
   auto mac = [&](acc_t a, acc_t b, acc_t c) -> acc_t {
     if constexpr (T::is_int) return c + a * b;
     else return __builtin_fmaf(a, b, c);
   };
-  const int kv = K / EPV;   // whole 16-byte pieces of a K line
-  for (int v = lane; v < kv; v += 64) {
-    const int k0 = v * EPV;
-    in_t a[EPV];
-    if constexpr (A_KC) {
-      __builtin_memcpy(a, g.A + (size_t)m * K + k0, 16);
-    } else {
+  for (int kc0 = 0; kc0 < K; kc0 += STRIP_K_CHUNK) {
+    const int kn = min(STRIP_K_CHUNK, K - kc0), kn_pad = (kn + EPV - 1) / EPV * EPV;   // zero-filled up to whole vectors
+    for (int j = 0; j < r; j++)
+      for (int k = threadIdx.x; k < kn_pad; k += STRIP_WAVES * 64)
+        bs[j * STRIP_K_CHUNK + k] = k < kn ? (B_KC ? g.B[(size_t)j * K + kc0 + k] : g.B[(size_t)(kc0 + k) * ldb + j]) : (in_t)0;
+    __syncthreads();
 #pragma unroll
-      for (int e = 0; e < EPV; e++) a[e] = g.A[(size_t)(k0 + e) * M + m];
-    }
-#pragma unroll
-    for (int j = 0; j < R; j++) {
-      if (j < r) {   // the same for every lane
-        in_t b[EPV];
-        if constexpr (B_KC) {
-          __builtin_memcpy(b, g.B + (size_t)j * K + k0, 16);
+    for (int i = 0; i < STRIP_ROWS_PER_WAVE; i++) {
+      const int m = m0 + i;
+      if (m >= M) break;
+      for (int k0 = lane * EPV; k0 < kn_pad; k0 += 64 * EPV) {
+        const int k = kc0 + k0;
+        in_t a[EPV];
+        if (A_KC && k + EPV <= K) {
+          __builtin_memcpy(a, g.A + (size_t)m * K + k, 16);
         } else {
 #pragma unroll
-          for (int e = 0; e < EPV; e++) b[e] = g.B[(size_t)(k0 + e) * ldb + j];
+          for (int e = 0; e < EPV; e++)
+            a[e] = k + e < K ? (A_KC ? g.A[(size_t)m * K + k + e] : g.A[(size_t)(k + e) * M + m]) : (in_t)0;
         }
 #pragma unroll
-        for (int e = 0; e < EPV; e++) acc[j] = mac(widen_in<TYPES>(a[e]), widen_in<TYPES>(b[e]), acc[j]);
+        for (int j = 0; j < R; j++) {
+          if (j < r) {   // the same for every lane
+            in_t b[EPV];
+            __builtin_memcpy(b, __builtin_assume_aligned(bs + j * STRIP_K_CHUNK + k0, 16), 16);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) acc[i][j] = mac(widen_in<TYPES>(a[e]), widen_in<TYPES>(b[e]), acc[i][j]);
+          }
+        }
       }
     }
-  }
-  const int k = kv * EPV + lane;   // what is left of a ragged K, one element per lane
-  if (k < K) {
-    const acc_t a = widen_in<TYPES>(A_KC ? g.A[(size_t)m * K + k] : g.A[(size_t)k * M + m]);
-#pragma unroll
-    for (int j = 0; j < R; j++)
-      if (j < r) acc[j] = mac(a, widen_in<TYPES>(B_KC ? g.B[(size_t)j * K + k] : g.B[(size_t)k * ldb + j]), acc[j]);
+    __syncthreads();
   }
 #pragma unroll
-  for (int j = 0; j < R; j++)
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) acc[j] += __shfl_xor(acc[j], off, 64);
-  if (lane == 0) {
+  for (int i = 0; i < STRIP_ROWS_PER_WAVE; i++) {
+    const int m = m0 + i;
+    if (m >= M) break;
 #pragma unroll
     for (int j = 0; j < R; j++) {
-      if (j < r) {
+      acc_t v = acc[i][j];
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+      if (lane == 0 && j < r) {
         const size_t o = (size_t)m * g.ldd + j;
-        g.D[o] = epilogue<TYPES>(acc[j], g.alpha, g.beta, g.C + o);
+        g.D[o] = epilogue<TYPES>(v, g.alpha, g.beta, g.C + o);
       }
     }
   }
 }
 
 template <int TYPES> static int launch_strip(const GemmArgs<TYPES>& g, hipStream_t s) {
-  const dim3 grid((unsigned)ceil_div(g.M, STRIP_ROWS_PER_WG)), block(STRIP_ROWS_PER_WG * 64);
+  const dim3 grid((unsigned)ceil_div(g.M, STRIP_ROWS_PER_WG)), block(STRIP_WAVES * 64);
   const bool akc = g.layoutA == GZ_ROW_MAJOR, bkc = g.layoutB == GZ_COL_MAJOR;
 #define GZ_STRIP(AKC, BKC)                                                                              \
   do {                                                                                                  \

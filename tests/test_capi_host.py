@@ -92,8 +92,8 @@ def test_plan_headline_configs(capi):
     assert (p.rung, p.tile_k, p.grid) == (capi.RUNG_MFMA, 128, 1024)
     # ragged fp16 problem: ceil-div grid, only 2-byte aligned lines
     p = capi.plan(capi.F16F16F16, 4095, 4097, 1023, 0, 0)
-    # the one column past 4096 runs as a second launch: dot products, one wave per row, four rows per work-group
-    assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n, p.tail_grid) == (1, 4, 1, 1024)
+    # the one column past 4096 runs as a second launch: dot products, one wave per row, sixteen rows per work-group
+    assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n, p.tail_grid) == (1, 16, 1, 256)
     assert p.grid == -(-4095 // p.tile_m) * (4096 // p.tile_n)
     assert p.vector_bytes_a == 2 and p.vector_bytes_b == 2
     # decode shapes go to the streaming kernel under AUTO, big M does not

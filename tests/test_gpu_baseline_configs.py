@@ -224,7 +224,7 @@ def test_columns_past_a_multiple_of_256_run_as_a_second_launch(G, types, shape):
         split_seen |= p.tail_cols > 0
         if p.tail_cols:
             assert p.tail_cols == n % 256 and p.tail_rows == 0
-            assert (p.tail_tile_m, p.tail_tile_n) == ((4, p.tail_cols) if p.tail_cols <= 8 else (128, 128))
+            assert (p.tail_tile_m, p.tail_tile_n) == ((16, p.tail_cols) if p.tail_cols <= 8 else (128, 128))
             assert p.grid == -(-m // p.tile_m) * ((n - p.tail_cols) // p.tile_n)
         a, b, c = O.make_inputs(types, m, n, k, kind=kind, seed=5 + la + 2 * lb)
         print("case", types, shape, la, lb, p.tail_cols, flush=True)
@@ -237,6 +237,6 @@ def test_columns_past_a_multiple_of_256_run_as_a_second_launch(G, types, shape):
 
 def test_ragged_baseline_shape_is_split_by_columns(G):
     p = G.capi.plan(O.F16F16F16, 4095, 4097, 1023, O.ROW, O.ROW)
-    assert (p.tile_m, p.tile_n, p.grid, p.tail_cols, p.tail_tile_m, p.tail_grid) == (256, 256, 256, 1, 4, 1024)
+    assert (p.tile_m, p.tile_n, p.grid, p.tail_cols, p.tail_tile_m, p.tail_grid) == (256, 256, 256, 1, 16, 256)
     assert G.capi.plan(O.F16F16F16, 4096, 4096, 1024, O.ROW, O.ROW).tail_cols == 0
     assert G.capi.plan(O.F16F16F16, 4096, 4096 + 100, 1024, O.ROW, O.ROW).tail_cols == 0
