@@ -117,7 +117,12 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
                                      : 0.40 + 0.27 * rounds + 0.035 * (rounds > 4 ? rounds - 4 : 0);
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
     const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : 1.15) : 1.0;
-    const double cost = shape_cost * rowb * (direct ? 1.0 : 2.2);
+    // what the register-staged kernel costs over a direct-to-LDS one on the same tile (4096 x 4096 x 4000 against
+    // 4096^3, us: bf16 256 x 256 on eight waves 134 / 117, 128 x 128 168 against an estimated 173; int8 82 / 69 and
+    // 104 / 102; fp8, four waves, 105 / 68.5 and 99 / 101); fp32 has no other kernel, its factor only weighs the splits
+    const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
+    const double staged = types == GZ_F32F32F32 ? 2.2 : i == 2 ? 1.05 : f8 ? (i == 0 ? 1.5 : 1.3) : 1.2;
+    const double cost = shape_cost * rowb * (direct ? 1.0 : staged);
     if (i == 0 || cost < best) {
       best = cost;
       pick = cand[i];
@@ -149,10 +154,13 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
 // (4096 x 4096 x 4000, us, four / eight waves: int8 96 / 82 and 103 / 84 with a row-major B, bf16 161 / 133 and
 // 180 / 149) and four for the 8-bit floats, whose eight-wave instance does not fit its registers (105 / 206).
 inline void mfma_adjust_general(int types, int cls, int layoutA, MfmaCfg* c) {
-  if (cls != MFMA_SHAPE_GENERAL || c->bm != 256 || c->bn != 256) return;
+  // (whole tiles of a column-major A are in the "whole" class and still run on that kernel; they gain as well:
+  // 4096^3, int8 84 / 77, bf16 135 / 124 and 144 / 128 with a row-major B)
+  const bool staged = cls == MFMA_SHAPE_GENERAL || layoutA != GZ_ROW_MAJOR;
+  if (!staged || c->bm != 256 || c->bn != 256) return;
   const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
   if (f8) *c = kMfmaCfgs[0];
-  else if (types != GZ_F32F32F32 && layoutA == GZ_ROW_MAJOR) *c = kMfmaCfgs[1];
+  else if (types != GZ_F32F32F32) *c = kMfmaCfgs[1];
 }
 
 // Ragged last round.  When the 256x256 tiles of a problem fill some rounds of the compute units and then leave a
@@ -221,7 +229,7 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   const bool direct_before = layoutA == GZ_ROW_MAJOR && types != GZ_F32F32F32 &&
                              (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && main_cfg.bm == 256 && main_cfg.bn == 256));
   const bool direct_after = direct_before && layoutB == GZ_COL_MAJOR && main_cfg.bm == 256 && main_cfg.bn == 256;
-  if (direct_before && !direct_after) cost_main *= 2.2;
+  if (direct_before && !direct_after) cost_main *= types == GZ_F32F32F32 ? 2.2 : mfma_in_size(types) == 2 ? 1.2 : 1.5;
   // on the register-staged kernel eight waves carry a 256 x 256 tile of 16-bit elements better than four
   // (fp16 4095 x 4097 x 1023, row-major B: 119 us against 158)
   if (!direct_after && main_cfg.bm == 256 && main_cfg.bn == 256 && mfma_in_size(types) == 2) main_cfg = kMfmaCfgs[6];

@@ -232,7 +232,9 @@ def test_columns_past_a_multiple_of_256_run_as_a_second_launch(G, types, shape):
         for rows in ((0, 24), (m - 24, m)):
             ref = O.gemm(types, a, b, c, m, n, k, la, lb, 2, -1, rows=rows)
             assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, shape, la, lb, rows)
-    assert split_seen
+    # (the 8-bit floats keep a strip of more than eight columns in the one launch: on their four-wave register-staged
+    # kernel the estimate prefers small tiles for everything)
+    assert split_seen or (types in O.FP8_TYPES and n % 256 > 8)
 
 
 def test_ragged_baseline_shape_is_split_by_columns(G):
