@@ -58,8 +58,8 @@ inline bool mfma_whole_tiles(const MfmaCfg& c, int in_size, int M, int N, int K)
 //     256x256   rounds                      one work-group per compute unit
 //     256x128   0.75 rounds                 one work-group per compute unit, more operand bytes per flop
 //     128x128   0.40 + 0.27 rounds          two work-groups share a compute unit; a lone one cannot fill it
-// (rounds = tiles of that size / compute units, rounded up), times 2.2 where the problem cannot use a direct-to-LDS
-// kernel, times 1.12 / 1.15 for the two smaller tiles on a row-major B (4096^3 row/row: 152 / 150 / 119).  A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does
+// (rounds = tiles of that size / compute units, rounded up), times the register-staged kernel's factor (see `staged` below) where the
+// problem cannot use a direct-to-LDS kernel, times 1.12 / 1.15 for the two smaller tiles on a row-major B (4096^3 row/row: 152 / 150 / 119).  A 256x256 tile needs the fewest bytes per flop and runs the hand-scheduled kernels, but a grid that does
 // not fill the device, or that leaves a nearly empty last round (N = 4097: 17 tile columns for one column of data),
 // is better served by smaller tiles.  Fitted to bf16 row/col squares, K = M = N (us, variants 3 / 4 / 6 =
 // 128x128 / 256x128 / 256x256):
