@@ -242,3 +242,47 @@ def test_ragged_baseline_shape_is_split_by_columns(G):
     assert (p.tile_m, p.tile_n, p.grid, p.tail_cols, p.tail_tile_m, p.tail_grid) == (256, 256, 256, 1, 16, 256)
     assert G.capi.plan(O.F16F16F16, 4096, 4096, 1024, O.ROW, O.ROW).tail_cols == 0
     assert G.capi.plan(O.F16F16F16, 4096, 4096 + 100, 1024, O.ROW, O.ROW).tail_cols == 0
+
+
+def random_big_problems(capi, types, want_cut=5, want_plain=2):
+    """Seeded draws of big problems with a short K; kept: the first `want_cut` that the launcher cuts in two launches
+    (rows or columns) and the first `want_plain` that it does not."""
+    rng = np.random.default_rng(77 + types)
+    es = np.dtype(O.IN_DTYPE[types]).itemsize
+    cut, plain = [], []
+    for _ in range(400):
+        m = int(rng.integers(2500, 7500))
+        n = 256 * int(rng.integers(10, 30)) + int(rng.choice([0, 0, 1, 3, 8, 9, 40, 64, 65, 130]))
+        k = (128 // es) * int(rng.integers(1, 3)) if rng.integers(0, 3) else int(rng.integers(24, 200))
+        la = O.ROW if rng.integers(0, 4) else O.COL
+        lb = int(rng.integers(0, 2))
+        al, be = int(rng.integers(1, 3)), int(rng.integers(-1, 2))
+        p = capi.plan(types, m, n, k, la, lb)
+        case = (m, n, k, la, lb, al, be, p.tail_rows, p.tail_cols)
+        if p.tail_rows or p.tail_cols:
+            if len(cut) < want_cut:
+                cut.append(case)
+        elif len(plain) < want_plain:
+            plain.append(case)
+        if len(cut) == want_cut and len(plain) == want_plain:
+            break
+    return cut, plain
+
+
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.F16F16F16])
+def test_launcher_choice_on_random_big_grids(G, types):
+    """Seeded random problems large enough for the launcher to cut them (a mostly empty last round of tiles: the
+    last rows in a second launch; a few columns past a multiple of 256: those columns in a second launch, as tiles
+    or as dot products), with a short K so that the oracle can follow: any layout, alpha and beta at work,
+    bit-exact on integer-valued data in the first and last rows and in a band around the cut."""
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+    cut, plain = random_big_problems(G.capi, types)
+    assert len(cut) >= 3, "the draw must exercise the cuts"
+    for m, n, k, la, lb, al, be, tail_rows, tail_cols in cut + plain:
+        a, b, c = O.make_inputs(types, m, n, k, kind=kind, seed=m + 3 * n + 5 * k)
+        print("case", types, m, n, k, la, lb, al, be, "tail_rows", tail_rows, "tail_cols", tail_cols, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, la, lb, al, be, -1)
+        edge = m - tail_rows if tail_rows else m // 2
+        for rows in ((0, 16), (max(edge - 8, 0), min(edge + 8, m)), (m - 16, m)):
+            ref = O.gemm(types, a, b, c, m, n, k, la, lb, al, be, rows=rows)
+            assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, m, n, k, la, lb, rows)
