@@ -285,14 +285,15 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       MfmaSplit sp;
       MfmaColSplit cs;
       int m_first = m, n_first = n;
-      if (variant == 0 && k > 0 && mfma_resolve_split(types, m, n, k, layoutA, layoutB, num_cus, &sp)) {
+      const int cut = (variant == 0 && k > 0) ? mfma_resolve_cut(types, m, n, k, layoutA, layoutB, num_cus, &sp, &cs) : 0;
+      if (cut == 1) {
         c = sp.main;
         m_first = sp.rows_main;
         plan->tail_rows = m - sp.rows_main;
         plan->tail_tile_m = sp.tail.bm;
         plan->tail_tile_n = sp.tail.bn;
         plan->tail_grid = (int64_t)ceil_div(m - sp.rows_main, sp.tail.bm) * ceil_div(n, sp.tail.bn);
-      } else if (variant == 0 && k > 0 && mfma_resolve_colsplit(types, m, n, k, layoutA, layoutB, num_cus, &cs)) {
+      } else if (cut == 2) {
         c = cs.main;
         n_first = cs.cols_main;
         plan->tail_cols = n - cs.cols_main;

@@ -173,7 +173,8 @@ struct MfmaSplit {
   int rows_main;      // rows of the first launch (a multiple of 256), 0 = no split
   MfmaCfg main, tail;
 };
-inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaSplit* out) {
+inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaSplit* out,
+                               double* estimate = nullptr) {
   out->rows_main = 0;
   if (num_cus <= 0) num_cus = 256;
   if (layoutA != GZ_ROW_MAJOR || M < 512 || N <= 0 || K <= 0) return false;
@@ -194,6 +195,7 @@ inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int 
     return false;
   const double cost_tail = mfma_choose(types, M - rows_main, N, K, layoutA, layoutB, num_cus, &tail_cfg);
   if (cost_main + cost_tail > 0.97 * cost_single) return false;
+  if (estimate) *estimate = cost_main + cost_tail;
   out->rows_main = rows_main;
   out->main = main_cfg;
   out->tail = tail_cfg;
@@ -214,7 +216,8 @@ struct MfmaColSplit {
   int cols_main;      // columns of the first launch (a multiple of 256), 0 = no split
   MfmaCfg main, tail;
 };
-inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaColSplit* out) {
+inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaColSplit* out,
+                                  double* estimate = nullptr) {
   out->cols_main = 0;
   if (num_cus <= 0) num_cus = 256;
   const int r = N % 256;
@@ -236,10 +239,22 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   tail_cfg = kMfmaCfgs[2];   // 128 x 128: the strip in as many work-groups as it has row blocks
   const double cost_tail = (r <= MFMA_STRIP_MAX_COLS ? 0.15 : 0.45) * ((M + 4095) / 4096);
   if (cost_main + cost_tail > 0.97 * cost_single) return false;
+  if (estimate) *estimate = cost_main + cost_tail;
   out->cols_main = cols_main;
   out->main = main_cfg;
   out->tail = tail_cfg;
   return true;
+}
+
+// Both cuts may apply to one problem (4096 x 4097: a 17th tile column that also spills into a second round): the one
+// with the lower estimate is taken.  Returns 0 (one launch), 1 (rows) or 2 (columns).
+inline int mfma_resolve_cut(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaSplit* rows,
+                            MfmaColSplit* cols) {
+  double est_rows = 0, est_cols = 0;
+  const bool by_rows = mfma_resolve_split(types, M, N, K, layoutA, layoutB, num_cus, rows, &est_rows);
+  const bool by_cols = mfma_resolve_colsplit(types, M, N, K, layoutA, layoutB, num_cus, cols, &est_cols);
+  if (by_rows && by_cols) return est_cols <= est_rows ? 2 : 1;
+  return by_rows ? 1 : by_cols ? 2 : 0;
 }
 
 // Shape class of a launch: the direct-to-LDS kernels also need 16-byte aligned operands.

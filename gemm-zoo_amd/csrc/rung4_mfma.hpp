@@ -216,17 +216,29 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         }
       });
     } else if constexpr (RAGGED) {
-      for (int r = 0; r < 32; r++) {
-        const int m = row0 + 32 * I + r;
-        if (m >= M) break;
-#pragma unroll
-        for (int c0 = 0; c0 < COLS; c0 += 64) {
-          const int nn = col0 + c0 + lane;
-          acc_t v;
-          __builtin_memcpy(&v, region + r * PITCH_E + (c0 + lane) * 4, 4);
-          const size_t o = (size_t)m * LDD + nn;
-          if (nn < N) g.D[o] = epilogue<TYPES>(v, g.alpha, g.beta, g.C + o);
-        }
+      // eight rows at a time: their LDS reads first, then the stores, so that a row does not wait for the one before
+      constexpr int RG = 8, NC = COLS / 64;
+      for (int r0 = 0; r0 < 32; r0 += RG) {
+        const int mg = row0 + 32 * I + r0;
+        if (mg >= M) break;
+        acc_t v[RG][NC];
+        static_for<RG>([&](auto r_c) {
+          constexpr int R = decltype(r_c)::value;
+          static_for<NC>([&](auto c_c) {
+            constexpr int C = decltype(c_c)::value;
+            __builtin_memcpy(&v[R][C], region + (r0 + R) * PITCH_E + (C * 64 + lane) * 4, 4);
+          });
+        });
+        static_for<RG>([&](auto r_c) {
+          constexpr int R = decltype(r_c)::value;
+          const int m = mg + R;
+          static_for<NC>([&](auto c_c) {
+            constexpr int C = decltype(c_c)::value;
+            const int nn = col0 + C * 64 + lane;
+            const size_t o = (size_t)m * LDD + nn;
+            if (m < M && nn < N) g.D[o] = epilogue<TYPES>(v[R][C], g.alpha, g.beta, g.C + o);
+          });
+        });
       }
     }
     // no wait here: the LDS executes a wave's instructions in order, so the next block's stores, issued right
@@ -1346,9 +1358,11 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
   GemmArgs<TYPES> g = args;
   g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), 256);
   if (variant == 0 && g.K > 0) {
-    // a mostly empty last round of 256x256 tiles: the rows that fill whole rounds first, the rest in a second launch
     MfmaSplit sp;
-    if (mfma_resolve_split(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, 256, &sp)) {
+    MfmaColSplit cs;
+    const int cut = mfma_resolve_cut(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, 256, &sp, &cs);
+    if (cut == 1) {
+      // a mostly empty last round of 256x256 tiles: the rows that fill whole rounds first, the rest in a second launch
       GemmArgs<TYPES> top = g, bottom = g;
       top.M = sp.rows_main;
       bottom.M = g.M - sp.rows_main;
@@ -1359,11 +1373,8 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       if (st != GZ_OK) return st;
       return launch_one<TYPES>(bottom, sp.tail, s, true);
     }
-  }
-  if (variant == 0 && g.K > 0) {
-    // a few columns past a multiple of 256: those columns in a launch of their own
-    MfmaColSplit cs;
-    if (mfma_resolve_colsplit(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, 256, &cs)) {
+    if (cut == 2) {
+      // a few columns past a multiple of 256: those columns in a launch of their own
       GemmArgs<TYPES> left = g, right = g;
       left.N = cs.cols_main;
       right.N = g.N - cs.cols_main;
