@@ -31,7 +31,10 @@ static const MfmaCfg kMfmaCfgs[] = {
 };
 constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
 
-inline int mfma_lds_bytes(const MfmaCfg& c) { return 2 * (c.bm + c.bn) * MFMA_LDS_PITCH; }
+// the most any kernel of the configuration asks for: the deep-pipeline kernels keep up to five buffers of 64-byte rows
+inline int mfma_lds_bytes(const MfmaCfg& c) {
+  return c.hand_scheduled == 2 ? 5 * (c.bm + c.bn) * 64 : 2 * (c.bm + c.bn) * MFMA_LDS_PITCH;
+}
 
 // How a problem sits on a tile configuration (16-byte alignment of the pointers is the caller's to check):
 //   WHOLE      whole tiles and whole K slabs

@@ -1113,6 +1113,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 }  // namespace gz
 
 #include "rung4_mfma_pipe4.hpp"
+#include "rung4_mfma_ring5.hpp"
 
 namespace gz {
 
@@ -1164,6 +1165,18 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   if (!edge && akc && bkc) {  // whole tiles, K-contiguous operands, aligned: direct-to-LDS fast path
     const size_t dlds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
     if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
+      if constexpr (!is_fp8(TYPES)) {
+        // K a whole number of 128-byte slabs: the variant whose copies ask for whole cache lines
+        if (hand_scheduled == 2 && ((size_t)g.K * sizeof(typename Traits<TYPES>::in_t)) % 128 == 0) {
+          auto kern = mfma_ring5_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
+          const size_t rlds = 5u * (size_t)(BM + BN) * 64;
+          GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)rlds));
+          hipLaunchKernelGGL(kern, grid, block, rlds, s, g, tiles_m, tiles_n);
+          GZ_HIP_TRY(hipGetLastError());
+          return GZ_OK;
+        }
+      }
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>;
         const size_t plds = 4u * (size_t)(BM + BN) * 64;
