@@ -9,14 +9,18 @@
 // what keeps one copy batch per MFMA step:
 //
 // Per slab j (groups 2j and 2j+1 in buffers (2j) % 5 and (2j+1) % 5), four MFMA steps:
-//   step 0 : MFMAs on (j, step 0); requests the fragments of (j, 1); issues the B rows of group 2j+3
-//   step 1 : MFMAs on (j, 1); requests (j, 2); issues the A rows of group 2j+4
-//   step 2 : MFMAs on (j, 2); requests (j, 3); issues the B rows of group 2j+4
+//   step 0 : MFMAs on (j, step 0); requests the fragments of (j, 1); issues the A rows of group 2j+4
+//   step 1 : MFMAs on (j, 1); requests (j, 2); issues the B rows of group 2j+4
+//   step 2 : MFMAs on (j, 2); requests (j, 3)
 //   barrier: lgkmcnt(0) - this wave has finished reading slab j, whose two buffers are free afterwards;
 //            vmcnt(n)   - this wave's copies of groups 2j+2 and 2j+3 have landed (the n of group 2j+4 may fly,
 //                         n = copies per wave and group)
-//   step 3 : MFMAs on (j, 3); requests (j+1, 0); issues the A rows of group 2j+5 into buffer (2j) % 5
-// One memory instruction follows each MFMA, as in mfma_pipe4_kernel.
+//   step 3 : MFMAs on (j, 3); requests (j+1, 0); issues all of group 2j+5 into buffer (2j) % 5, which the barrier
+//            has just freed: the odd group has the shortest way to the barrier that needs it (three steps), so it
+//            goes out at once, up to two memory instructions after an MFMA
+// Elsewhere one memory instruction follows each MFMA, as in mfma_pipe4_kernel.  (EARLY_ODD = false spreads the
+// odd group over step 3 and the next step 0 instead, one instruction per MFMA throughout: 0.7-0.9 % slower with
+// eight waves, bf16 4096^3 108.8 against 107.9 us, 8192^3 792 against 785; no difference with four.)
 //
 // LDS: a copy fills 1 KiB with 8 rows of 128 bytes; 16-byte piece c of the row with index i (0..7) within its
 // copy and group parity p lives at slot c ^ i ^ p, so that the 16 rows which 16 consecutive lanes of a fragment
@@ -25,9 +29,13 @@
 // Whole tiles, K a multiple of the slab (128 bytes), A row-major and B column-major only.
 #pragma once
 
+#ifndef GZ_RING5_EARLY_ODD
+#define GZ_RING5_EARLY_ODD true
+#endif
+
 namespace gz {
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY_ODD = GZ_RING5_EARLY_ODD>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_ring5_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
@@ -123,30 +131,38 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 
   // One MFMA step: NMMA MFMAs on register set SET; after MFMA q the q-th memory instruction of the step:
   // first the NRD fragment reads of (ring position RJ, step RKS) into the other set, then this step's copies
-  // (the A or B rows of group c, parity CP, into buffer cst).
-  auto step = [&](auto set_c, auto rj_c, auto rks_c, auto copy_is_a, auto cp_c, int cst, int c, uint64_t cmask) {
+  // (the A rows, the B rows or both of group c, parity CP, into buffer cst).
+  auto step = [&](auto set_c, auto rj_c, auto rks_c, auto kind_c, auto cp_c, int cst, int c, uint64_t cmask) {
     constexpr int SET = decltype(set_c)::value;
-    constexpr bool IS_A = decltype(copy_is_a)::value;
-    constexpr int NC = IS_A ? A_PW : B_PW;
-    constexpr int NOPS = NRD + NC;
-    static_assert(NOPS <= NMMA, "one memory instruction per MFMA");
+    constexpr int KIND = decltype(kind_c)::value;   // copies of this step: 0 none, 1 A rows, 2 B rows, 3 both
+    constexpr int NA = (KIND & 1) ? A_PW : 0, NB = (KIND & 2) ? B_PW : 0;
+    constexpr int NOPS = NRD + NA + NB;
+    constexpr int PER = (NOPS + NMMA - 1) / NMMA;
+    static_assert(PER <= 2, "at most two memory instructions per MFMA");
     asm volatile("s_waitcnt lgkmcnt(0)");
-    if constexpr (IS_A) copy_a_begin(cst);
-    else copy_b_begin(cst);
+    if constexpr (NA > 0) copy_a_begin(cst);
+    else if constexpr (NB > 0) copy_b_begin(cst);
     static_for<NMMA>([&](auto q_c) {
       constexpr int Q = decltype(q_c)::value;
       asm_mfma32<TYPES>(acc[Q / FN][Q % FN], bf[SET][Q % FN], af[SET][Q / FN]);
-      if constexpr (Q < NRD) {
-        read_one(std::integral_constant<int, SET ^ 1>{}, q_c, rj_c, rks_c);
-      } else if constexpr (Q < NOPS) {
-        if constexpr (IS_A) copy_a(std::integral_constant<int, Q - NRD>{}, cp_c, c, cmask);
-        else copy_b(std::integral_constant<int, Q - NRD>{}, cp_c, c, cmask);
-      }
+      static_for<PER>([&](auto o_c) {
+        constexpr int OP = Q * PER + decltype(o_c)::value;
+        if constexpr (OP < NRD) {
+          read_one(std::integral_constant<int, SET ^ 1>{}, std::integral_constant<int, OP>{}, rj_c, rks_c);
+        } else if constexpr (OP < NRD + NA) {
+          copy_a(std::integral_constant<int, OP - NRD>{}, cp_c, c, cmask);
+        } else if constexpr (OP < NOPS) {
+          if constexpr (NA > 0 && OP == NRD + NA) copy_b_begin(cst);
+          copy_b(std::integral_constant<int, OP - NRD - NA>{}, cp_c, c, cmask);
+        }
+      });
     });
   };
 
-  const std::true_type is_a{};
-  const std::false_type is_b{};
+  const std::integral_constant<int, 0> no_copy{};
+  const std::integral_constant<int, 1> is_a{};
+  const std::integral_constant<int, 2> is_b{};
+  const std::integral_constant<int, 3> a_and_b{};
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
@@ -157,8 +173,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     return ((uint64_t)w << 32) | w;
   };
 
-  // ---- prologue: groups 0, 1, 2 whole and the A rows of 3 ----
-  static_for<3>([&](auto c_c) {
+  // ---- prologue: groups 0, 1, 2 whole and (EARLY_ODD: all of) the A rows of 3 ----
+  static_for<EARLY_ODD ? 4 : 3>([&](auto c_c) {
     constexpr int C = decltype(c_c)::value;
     const uint64_t m = mask_if(C < nc);
     copy_a_begin(C);
@@ -166,13 +182,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     copy_b_begin(C);
     static_for<B_PW>([&](auto t) { copy_b(t, std::integral_constant<int, C & 1>{}, C, m); });
   });
-  copy_a_begin(3);
-  {
+  if constexpr (!EARLY_ODD) {
+    copy_a_begin(3);
     const uint64_t m3 = mask_if(3 < nc);
     static_for<A_PW>([&](auto t) { copy_a(t, I1{}, 3, m3); });
   }
-  // slab 0 (groups 0 and 1) has landed; group 2 and the A rows of 3 may still be on their way
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(NCP + A_PW) : "memory");
+  // slab 0 (groups 0 and 1) has landed; what was issued after it may still be on its way
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(EARLY_ODD ? 2 * NCP : NCP + A_PW) : "memory");
   static_for<NRD>([&](auto r) { read_one(I0{}, r, I0{}, I0{}); });
 
   // ---- one slab; JR = j % 5 at compile time ----
@@ -181,16 +197,23 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     using NEXT = std::integral_constant<int, (JR + 1) % NST>;
     const int c3 = 2 * j + 3, c4 = 2 * j + 4, c5 = 2 * j + 5;
     const uint64_t m4 = mask_if(c4 < nc);
-    step(I0{}, jr_c, I1{}, is_b, I1{}, (2 * JR + 3) % NST, c3, mask_if(c3 < nc));
-    step(I1{}, jr_c, I2{}, is_a, I0{}, (2 * JR + 4) % NST, c4, m4);
-    step(I0{}, jr_c, I3{}, is_b, I0{}, (2 * JR + 4) % NST, c4, m4);
+    if constexpr (EARLY_ODD) {
+      step(I0{}, jr_c, I1{}, is_a, I0{}, (2 * JR + 4) % NST, c4, m4);
+      step(I1{}, jr_c, I2{}, is_b, I0{}, (2 * JR + 4) % NST, c4, m4);
+      step(I0{}, jr_c, I3{}, no_copy, I0{}, 0, 0, m4);
+    } else {
+      step(I0{}, jr_c, I1{}, is_b, I1{}, (2 * JR + 3) % NST, c3, mask_if(c3 < nc));
+      step(I1{}, jr_c, I2{}, is_a, I0{}, (2 * JR + 4) % NST, c4, m4);
+      step(I0{}, jr_c, I3{}, is_b, I0{}, (2 * JR + 4) % NST, c4, m4);
+    }
     if (c4 < nc) {  // the copies of group 2j+4 may stay in flight
       if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
-    step(I1{}, NEXT{}, I0{}, is_a, I1{}, (2 * JR + 5) % NST, c5, mask_if(c5 < nc));
+    if constexpr (EARLY_ODD) step(I1{}, NEXT{}, I0{}, a_and_b, I1{}, (2 * JR + 5) % NST, c5, mask_if(c5 < nc));
+    else step(I1{}, NEXT{}, I0{}, is_a, I1{}, (2 * JR + 5) % NST, c5, mask_if(c5 < nc));
   };
 
   const int nslab = nc / 2;
