@@ -1221,6 +1221,17 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
       GZ_HIP_TRY(hipGetLastError());
       return GZ_OK;
     }
+    if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2 && !is_fp8(TYPES)) {
+      if (hand_scheduled == 2 && ((size_t)g.K * sizeof(typename Traits<TYPES>::in_t)) % 128 == 0) {
+        auto kern = mfma_ring5_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;
+        const size_t rlds = 5u * (size_t)(BM + BN) * 64;
+        GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)rlds));
+        hipLaunchKernelGGL(kern, grid, block, rlds, s, g, tiles_m, tiles_n);
+        GZ_HIP_TRY(hipGetLastError());
+        return GZ_OK;
+      }
+    }
     if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2) {
       if (hand_scheduled == 2) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>;

@@ -26,7 +26,10 @@
 // copy and group parity p lives at slot c ^ i ^ p, so that the 16 rows which 16 consecutive lanes of a fragment
 // read touch fall into the 16 four-bank groups of a 64-bank line.
 //
-// Whole tiles, K a multiple of the slab (128 bytes), A row-major and B column-major only.
+// Whole tiles, K a multiple of the slab (128 bytes), A row-major.  B_KC = false: B is row-major; its copies move
+// whole K rows already, so group c simply carries K rows [h c, h c + h) of B (h = 32 16-bit or 64 int8 rows) in
+// mfma_pipe4_kernel's layout, read through the transposing LDS reads: MFMA step s of a slab finds its B rows in the
+// group of parity s / 2.
 #pragma once
 
 #ifndef GZ_RING5_EARLY_ODD
@@ -35,7 +38,7 @@
 
 namespace gz {
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY_ODD = GZ_RING5_EARLY_ODD>
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true, bool EARLY_ODD = GZ_RING5_EARLY_ODD>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_ring5_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
@@ -48,7 +51,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr int NST = 5;              // LDS buffers, one copy group each
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int FM = WM / 32, FN = WN / 32;
-  constexpr int NMMA = FM * FN, NRD = FM + FN;  // LDS reads per MFMA step
+  constexpr int EPV = 16 / ES;
+  constexpr int HK = 64 / ES;         // K rows of a row-major B per copy group
+  constexpr int NMMA = FM * FN, NRD = B_KC ? FM + FN : FM + 2 * FN;  // LDS reads per MFMA step
   constexpr int A_BYTES = BM / 2 * LINE, B_BYTES = BN / 2 * LINE;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (8 rows) per wave and group
@@ -76,7 +81,27 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   const uint32_t voff[2] = {(uint32_t)(ci * K * ES + ((cs ^ ci) * 16)), (uint32_t)(ci * K * ES + ((cs ^ ci ^ 1) * 16))};
   const size_t group_step = (size_t)16 * K * ES, parity_step = (size_t)8 * K * ES;
   const char* a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(m0 + 16 * wave * A_PW) * K * ES;
-  const char* b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 16 * wave * B_PW) * K * ES;
+  // row-major B: group c carries K rows [HK c, HK c + HK) of B, BN elements each, as mfma_pipe4_kernel lays them out:
+  // a copy moves KRC whole K rows; lane -> (row, 16-byte position), pieces of K row r at position piece ^ f(r)
+  constexpr int KRC = 1024 / (BN * ES), LPR = 64 / KRC;
+  const int N = g.N;
+  uint32_t voff_b[2] = {0, 0};
+  const char* b_ubase;
+  size_t b_copy_step = 0, b_group_step = 0;
+  if constexpr (B_KC) {
+    b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 16 * wave * B_PW) * K * ES;
+  } else {
+    static_assert(B_KC || (KRC * BN * ES == 1024 && B_PW % 2 == 0), "whole K rows per copy");
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+      const int kr = KRC * par + lane / LPR;
+      const int f = ES == 2 ? (kr & 3) << 2 : (kr & 7) << 1;
+      voff_b[par] = (uint32_t)(((size_t)(lane / LPR) * N + (size_t)(((lane % LPR) ^ f) * EPV)) * ES);
+    }
+    b_ubase = reinterpret_cast<const char*>(g.B) + ((size_t)(wave * B_PW * KRC) * N + n0) * ES;
+    b_copy_step = (size_t)KRC * N * ES;
+    b_group_step = (size_t)HK * N * ES;
+  }
   auto copy_a_begin = [&](int st) { asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024); };
   auto copy_b_begin = [&](int st) {
     asm_set_m0(lds_base + st * STAGE_BYTES + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024);
@@ -88,14 +113,15 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   };
   auto copy_b = [&](auto t_c, auto p_c, int c, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - B_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(voff[P], b_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
+    if constexpr (B_KC) asm_copy16_masked<OFF>(voff[P], b_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
+    else asm_copy16_masked<OFF>(voff_b[Tn & 1], b_ubase + Tn * b_copy_step + (size_t)c * b_group_step - OFF, mask);
   };
 
   // ---- fragment addressing: one LDS byte address per (slab position in the ring, step) ----
   // tile row r = 16 G + 8 p + i lives in the buffer of group parity p at G * 1024 + i * 128
   const int frag_row = lane & 31, half = lane >> 5;
   const int fp = (frag_row >> 3) & 1, fi = frag_row & 7;
-  uint32_t a_addr[NST][4], b_addr[NST][4];
+  uint32_t a_addr[NST][4], b_addr[NST][B_KC ? 4 : FN];  // row-major B: per (buffer, 32-column block)
 #pragma unroll
   for (int jr = 0; jr < NST; jr++) {
     const int buf = (2 * jr + fp) % NST;
@@ -103,8 +129,31 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     for (int ks = 0; ks < 4; ks++) {
       const int pos = ((ks * 2 + half) ^ fi ^ fp) * 16;
       a_addr[jr][ks] = lds_base + buf * STAGE_BYTES + (wm * WM / 16 + (frag_row >> 4)) * 1024 + fi * LINE + pos;
-      b_addr[jr][ks] = lds_base + buf * STAGE_BYTES + A_BYTES + (wn * WN / 16 + (frag_row >> 4)) * 1024 + fi * LINE + pos;
+      if constexpr (B_KC)
+        b_addr[jr][ks] = lds_base + buf * STAGE_BYTES + A_BYTES + (wn * WN / 16 + (frag_row >> 4)) * 1024 + fi * LINE + pos;
     }
+  }
+
+  // transposing reads of a row-major B (see mfma_pipe4_kernel): one address per (buffer, 32-column block); K step
+  // within the group and half fragment go into the immediate offset
+  constexpr int TR_LPR = ES == 2 ? 4 : 2;
+  constexpr int TR_PITCH = BN * ES;
+  constexpr int TR_KS_OFF = (16 / ES * 2) * TR_PITCH;
+  constexpr int TR_R_OFF = (16 / TR_LPR) * TR_PITCH;
+  if constexpr (!B_KC) {
+    static_assert(B_KC || (TR_KS_OFF + TR_R_OFF < 65536 && TR_KS_OFF == B_BYTES / 2), "immediate offsets");
+    const int i16 = lane & 15, ti = i16 / TR_LPR;
+    const int n_sub = ((lane >> 4) & 1) * 16 + (i16 % TR_LPR) * (8 / ES);
+    const int krow = (lane >> 5) * (16 / TR_LPR * 2) + ti;
+    const int f = ES == 2 ? (ti & 3) << 2 : (ti & 7) << 1;
+#pragma unroll
+    for (int st = 0; st < NST; st++)
+#pragma unroll
+      for (int j = 0; j < FN; j++) {
+        const int n_local = wn * WN + j * 32 + n_sub;
+        const int piece = (n_local / EPV) ^ f;
+        b_addr[st][j] = lds_base + st * STAGE_BYTES + A_BYTES + krow * TR_PITCH + piece * 16 + (n_local % EPV) * ES;
+      }
   }
 
   acc_v acc[FM][FN];
@@ -120,13 +169,18 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   });
   asm volatile("s_nop 7" ::: "memory");
   u32x4_t af[2][FM], bf[2][FN];  // register sets of fragments: one per MFMA step, alternating
+  u32x2_t bh[2][FN][2];          // row-major B: the two halves of a fragment as they come out of the transposing reads
 
   // 32 rows of a fragment are two 16-row groups: 2 KiB per fragment
   auto read_one = [&](auto set_c, auto r_c, auto jr_c, auto ks_c) {
     constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value;
     constexpr int JR = decltype(jr_c)::value, KS = decltype(ks_c)::value;
     if constexpr (R < FM) asm_ds_read16<R * 2048>(af[SET][R], a_addr[JR][KS]);
-    else asm_ds_read16<(R - FM) * 2048>(bf[SET][R - FM], b_addr[JR][KS]);
+    else if constexpr (B_KC) asm_ds_read16<(R - FM) * 2048>(bf[SET][R - FM], b_addr[JR][KS]);
+    else {  // K rows 16 KS .. of the slab sit in the group of parity KS / 2, at its local step KS % 2
+      constexpr int J = (R - FM) / 2, HALF = (R - FM) % 2, ST = (2 * JR + KS / 2) % NST;
+      asm_ds_read_tr<ES, (KS % 2) * TR_KS_OFF + HALF * TR_R_OFF>(bh[SET][J][HALF], b_addr[ST][J]);
+    }
   };
 
   // One MFMA step: NMMA MFMAs on register set SET; after MFMA q the q-th memory instruction of the step:
@@ -140,6 +194,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     constexpr int PER = (NOPS + NMMA - 1) / NMMA;
     static_assert(PER <= 2, "at most two memory instructions per MFMA");
     asm volatile("s_waitcnt lgkmcnt(0)");
+    if constexpr (!B_KC) {
+#pragma unroll
+      for (int j = 0; j < FN; j++) {
+        asm volatile("" : "+v"(bh[SET][j][0]), "+v"(bh[SET][j][1]));  // after the wait
+        bf[SET][j] = u32x4_t{bh[SET][j][0][0], bh[SET][j][0][1], bh[SET][j][1][0], bh[SET][j][1][1]};
+      }
+    }
     if constexpr (NA > 0) copy_a_begin(cst);
     else if constexpr (NB > 0) copy_b_begin(cst);
     static_for<NMMA>([&](auto q_c) {
