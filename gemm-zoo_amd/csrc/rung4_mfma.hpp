@@ -1145,6 +1145,17 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
   if (shape_class == MFMA_SHAPE_RAGGED_MN && akc && hand_scheduled == 2) {
     if constexpr (PIPE4 && BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4)) {
       const size_t plds = 4u * (size_t)(BM + BN) * 64;
+      if constexpr (!is_fp8(TYPES)) {
+        if (bkc) {   // the shape class says whole K slabs: the whole-line kernel, rows clamped
+          auto kern = mfma_ring5_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>;
+          const size_t rlds = 5u * (size_t)(BM + BN) * 64;
+          GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)rlds));
+          hipLaunchKernelGGL(kern, grid, block, rlds, s, g, tiles_m, tiles_n);
+          GZ_HIP_TRY(hipGetLastError());
+          return GZ_OK;
+        }
+      }
       if (bkc) {
         auto kern = mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>;
         GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

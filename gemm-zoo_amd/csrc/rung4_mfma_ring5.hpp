@@ -26,7 +26,8 @@
 // copy and group parity p lives at slot c ^ i ^ p, so that the 16 rows which 16 consecutive lanes of a fragment
 // read touch fall into the 16 four-bank groups of a 64-bank line.
 //
-// Whole tiles, K a multiple of the slab (128 bytes), A row-major.  B_KC = false: B is row-major; its copies move
+// K a multiple of the slab (128 bytes), A row-major; whole tiles, or (RAGGED, column-major B) any M and N with
+// 16-byte aligned rows.  B_KC = false: B is row-major; its copies move
 // whole K rows already, so group c simply carries K rows [h c, h c + h) of B (h = 32 16-bit or 64 int8 rows) in
 // mfma_pipe4_kernel's layout, read through the transposing LDS reads: MFMA step s of a slab finds its B rows in the
 // group of parity s / 2.
@@ -38,7 +39,7 @@
 
 namespace gz {
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true, bool EARLY_ODD = GZ_RING5_EARLY_ODD>
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool B_KC = true, bool RAGGED = false, bool EARLY_ODD = GZ_RING5_EARLY_ODD>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_ring5_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
@@ -59,6 +60,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (8 rows) per wave and group
   constexpr int NCP = A_PW + B_PW;
   static_assert(!is_fp8(TYPES) && TYPES != GZ_F32F32F32, "16-bit and int8 operands");
+  static_assert(B_KC || !RAGGED, "ragged grids with a column-major B only");
   static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile rows must divide over the waves");
   static_assert(A_PW <= 8 && B_PW <= 8 && A_PW % 2 == 0 && B_PW % 2 == 0, "a copy group must fit the immediate offset range");
   static_assert(NCP == 8 || NCP == 4, "the vmcnt immediates below are written out for 8 or 4 copies per wave and group");
@@ -102,6 +104,27 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     b_copy_step = (size_t)KRC * N * ES;
     b_group_step = (size_t)HK * N * ES;
   }
+  // RAGGED: M and N need not be multiples of the tile.  Rows past the end are fetched from the last row: an output
+  // depends on its own row of A and column of B only, and those past the end are not stored.  The per-copy offsets
+  // are then relative to the tile's first row instead of the copy's.
+  uint32_t voff_ar[2][RAGGED ? A_PW : 1], voff_br[2][RAGGED ? B_PW : 1];
+  const char* a_tile = reinterpret_cast<const char*>(g.A) + (size_t)m0 * K * ES;
+  const char* b_tile = reinterpret_cast<const char*>(g.B) + (size_t)n0 * K * ES;
+  if constexpr (RAGGED) {
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+#pragma unroll
+      for (int t = 0; t < A_PW; t++) {
+        const int rc = min(m0 + 16 * (wave * A_PW + t) + 8 * par + ci, g.M - 1) - m0;
+        voff_ar[par][t] = (uint32_t)((size_t)rc * K * ES + (size_t)((cs ^ ci ^ par) * 16));
+      }
+#pragma unroll
+      for (int t = 0; t < B_PW; t++) {
+        const int rc = min(n0 + 16 * (wave * B_PW + t) + 8 * par + ci, g.N - 1) - n0;
+        voff_br[par][t] = (uint32_t)((size_t)rc * K * ES + (size_t)((cs ^ ci ^ par) * 16));
+      }
+    }
+  }
   auto copy_a_begin = [&](int st) { asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024); };
   auto copy_b_begin = [&](int st) {
     asm_set_m0(lds_base + st * STAGE_BYTES + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024);
@@ -109,11 +132,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // copy t of this wave for group c (parity P = c & 1 at compile time)
   auto copy_a = [&](auto t_c, auto p_c, int c, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - A_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(voff[P], a_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
+    if constexpr (RAGGED) asm_copy16_masked<OFF>(voff_ar[P][Tn], a_tile + (size_t)(c >> 1) * LINE - OFF, mask);
+    else asm_copy16_masked<OFF>(voff[P], a_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
   };
   auto copy_b = [&](auto t_c, auto p_c, int c, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - B_PW / 2) * 1024;
-    if constexpr (B_KC) asm_copy16_masked<OFF>(voff[P], b_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
+    if constexpr (RAGGED) asm_copy16_masked<OFF>(voff_br[P][Tn], b_tile + (size_t)(c >> 1) * LINE - OFF, mask);
+    else if constexpr (B_KC) asm_copy16_masked<OFF>(voff[P], b_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
     else asm_copy16_masked<OFF>(voff_b[Tn & 1], b_ubase + Tn * b_copy_step + (size_t)c * b_group_step - OFF, mask);
   };
 
@@ -296,7 +321,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 
   static_assert(NW * epilogue_region_bytes<FN>() <= NST * STAGE_BYTES, "the epilogue reuses the operand buffers");
   __syncthreads();   // no wave reads operands any more and no copy is in flight
-  store_accumulators_lds<TYPES, FM, FN, false>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
+  store_accumulators_lds<TYPES, FM, FN, RAGGED>(g, acc, m0 + wm * WM, n0 + wn * WN, lane, lds + wave * epilogue_region_bytes<FN>());
 }
 
 }  // namespace gz

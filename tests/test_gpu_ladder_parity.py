@@ -89,6 +89,19 @@ def test_whole_line_pipeline_every_slab_count(G, types):
         print("case", types, variant, m, n, k, flush=True)
         got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1, MFMA, variant)
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1)), (types, variant, m, n, k)
+    # ragged M and N with whole slabs (rows clamped at the edges), and a row-major B on whole tiles (variant 6)
+    for variant, slabs, (m, n) in itertools.product((6, 7), (1, 4, 7), [(300, 520), (257, 255), (511, 1)]):
+        k = slab * slabs
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs + 50)
+        print("ragged case", types, variant, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1)), (types, variant, m, n, k)
+    for slabs, (m, n) in itertools.product((1, 2, 5, 6, 11), [(256, 512)]):
+        k = slab * slabs
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs + 90)
+        print("row/row case", types, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1, MFMA, 6)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1)), (types, m, n, k)
 
 
 @pytest.mark.parametrize("types", ALL_TYPES)
