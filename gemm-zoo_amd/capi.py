@@ -21,6 +21,11 @@ RUNG_AUTO, RUNG_NAIVE, RUNG_COALESCED, RUNG_LDS_TILED, RUNG_DOUBLE_BUFFERED, RUN
 NUM_RUNGS = 6
 DT_INT8, DT_BF16, DT_F16, DT_F32, DT_INT32, DT_E4M3, DT_E5M2 = 0, 1, 2, 3, 4, 5, 6
 FILL_INT8_UNIFORM, FILL_NORMAL, FILL_UNIFORM_PM1, FILL_SMALL_INT = 0, 1, 2, 3
+# tile configurations of the MFMA rung (variant ids; 0 = the launcher chooses): the register-staged / compiler-scheduled
+# kernels on four tiles, the hand-scheduled ring kernel on four and eight waves, the same with the stream-K
+# decomposition, and the ring kernel with one work-group per tile instead of one per compute unit
+MFMA_256_W4, MFMA_256_W8, MFMA_128, MFMA_256X128 = 1, 2, 3, 4
+MFMA_RING_W4, MFMA_RING_W8, MFMA_STREAMK_W4, MFMA_STREAMK_W8, MFMA_RING_W4_PER_TILE, MFMA_RING_W8_PER_TILE = 5, 6, 7, 8, 9, 10
 
 TYPES_NAMES = {S8S8S32: "s8s8s32", BF16BF16F32: "bf16bf16f32", BF16BF16BF16: "bf16bf16bf16", F16F16F16: "f16f16f16",
                F32F32F32: "f32f32f32", E4M3E4M3F16: "e4m3e4m3f16", E5M2E5M2F16: "e5m2e5m2f16",
@@ -34,7 +39,7 @@ EXPORTS = [
     "gz_gemm_s8s8s32", "gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16", "gz_gemm_f32f32f32",
     "gz_gemm_e4m3e4m3f16", "gz_gemm_e5m2e5m2f16", "gz_gemm_bf16bf16bf16_acc16", "gz_gemm_f16f16f16_acc16", "gz_gemm",
     "gz_plan", "gz_variant_count", "gz_rung_name", "gz_types_name", "gz_fill", "gz_compare", "gz_compare_rel",
-    "gz_last_error", "gz_version", "gz_device_props", "gz_gemm_static_scratch",
+    "gz_last_error", "gz_version", "gz_device_props", "gz_gemm_static_scratch", "gz_plan_static_scratch",
 ]
 
 
@@ -79,6 +84,7 @@ def _load():
     lib.gz_gemm.argtypes = [i32] + common + [f64, f64, i32, i32, vp]
     lib.gz_gemm_static_scratch.argtypes = [i32] + common + [f64, f64, i32, i32, vp]
     lib.gz_plan.argtypes = [i32, i64, i64, i64, i32, i32, i32, i32, i32, i32, C.POINTER(Plan)]
+    lib.gz_plan_static_scratch.argtypes = lib.gz_plan.argtypes
     lib.gz_variant_count.argtypes = [i32, i32]
     lib.gz_rung_name.argtypes = [i32]
     lib.gz_rung_name.restype = C.c_char_p
@@ -147,6 +153,14 @@ def plan(types: int, m: int, n: int, k: int, layout_a: int = ROW_MAJOR, layout_b
          rung: int = RUNG_AUTO, variant: int = 0, num_cus: int = 0, lds_per_cu: int = 0) -> Plan:
     p = Plan()
     check(lib.gz_plan(types, m, n, k, layout_a, layout_b, rung, variant, num_cus, lds_per_cu, C.byref(p)))
+    return p
+
+
+def plan_static_scratch(types: int, m: int, n: int, k: int, layout_a: int = ROW_MAJOR, layout_b: int = ROW_MAJOR,
+                        rung: int = RUNG_AUTO, variant: int = 0, num_cus: int = 0, lds_per_cu: int = 0) -> Plan:
+    """The plan gz_gemm_static_scratch takes: gz_plan within the static scratch buffer."""
+    p = Plan()
+    check(lib.gz_plan_static_scratch(types, m, n, k, layout_a, layout_b, rung, variant, num_cus, lds_per_cu, C.byref(p)))
     return p
 
 

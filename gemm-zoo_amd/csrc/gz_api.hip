@@ -61,11 +61,13 @@ std::mutex g_pool_mutex;
 std::map<std::pair<int, hipStream_t>, PoolBuffer> g_pool;   // never freed before the process ends
 }  // namespace
 
+size_t workspace_limit() { return t_static_scratch ? (size_t)GZ_STATIC_SCRATCH_BYTES : ~(size_t)0; }
+
 int workspace_acquire(size_t bytes, hipStream_t s, void** out) {
   if (t_static_scratch) {   // no allocation on this path
     if (bytes > (size_t)GZ_STATIC_SCRATCH_BYTES) {
       set_error("this launch needs %zu bytes of scratch memory, the static buffer holds %lld: use gz_gemm, which "
-                "allocates what it needs, or a variant without stream-K (8, 9)", bytes,
+                "allocates what it needs, or a variant without stream-K (5, 6)", bytes,
                 (long long)GZ_STATIC_SCRATCH_BYTES);
       return GZ_ERR_UNSUPPORTED;
     }
@@ -334,8 +336,10 @@ int gz_variant_count(int types, int rung) {
   }
 }
 
-int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung, int variant, int num_cus,
-            int lds_per_cu, gz_plan_t* plan) {
+// ws_limit: the most device memory beyond the matrices that the launch may use (what workspace_limit() will say
+// inside the entry point the plan is asked for)
+static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung, int variant,
+                     int num_cus, int lds_per_cu, size_t ws_limit, gz_plan_t* plan) {
   if (!plan) { set_error("plan is NULL"); return GZ_ERR_BAD_ARG; }
   int st = check_problem(types, M, N, K, layoutA, layoutB, rung);
   if (st != GZ_OK) return st;
@@ -387,12 +391,13 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
         plan->grid = (int64_t)ceil_div(m, 128) * ceil_div(n, 128);
         return GZ_OK;
       }
-      if ((variant == 0 || variant == 10 || variant == 11) && k > 0) {   // as launch_mfma, aligned operands assumed
+      if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && k > 0) {   // as launch_mfma, aligned operands assumed
         StreamKPlan skp;
         const MfmaCfg* forced = variant == 0 ? nullptr : &kMfmaCfgs[variant - 1];
-        if (mfma_plan_streamk(types, m, n, k, layoutA, layoutB, num_cus, forced != nullptr, forced, &skp)) {
+        if (mfma_plan_streamk(types, m, n, k, layoutA, layoutB, num_cus, forced != nullptr, forced, &skp) &&
+            (forced || (size_t)skp.slots * MFMA_STREAMK_SLOT_BYTES <= ws_limit)) {
           const MfmaCfg& c = skp.cfg;
-          plan->variant = c.waves_n == 4 ? 11 : 10;
+          plan->variant = c.waves_n == 4 ? MFMA_VARIANT_STREAMK_W8 : MFMA_VARIANT_STREAMK_W4;
           plan->tile_m = c.bm; plan->tile_n = c.bn; plan->tile_k = MFMA_SLAB_BYTES / es;
           plan->wave_m = c.bm / c.waves_m; plan->wave_n = c.bn / c.waves_n;
           plan->threads = c.waves_m * c.waves_n * 64;
@@ -449,7 +454,7 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
       plan->lds_bytes = mfma_lds_bytes(c);
       plan->grid = (int64_t)ceil_div(m_first, c.bm) * ceil_div(n_first, c.bn);
       // whole tiles on the ring kernel with the 16x16 instructions: one work-group per compute unit walks the tiles
-      if (c.hand_scheduled >= 3 && types != GZ_F32F32F32 && layoutA == GZ_ROW_MAJOR &&
+      if (c.ring == 1 && types != GZ_F32F32F32 && layoutA == GZ_ROW_MAJOR &&
           mfma_shape_class(c, es, m_first, n_first, k, layoutA, layoutB) == MFMA_SHAPE_WHOLE)
         plan->grid = mfma_persistent_grid(plan->grid, num_cus);
       if (plan->lds_bytes > lds_per_cu) {
@@ -478,6 +483,17 @@ int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB
   }
   set_error("unknown rung %d", rung);
   return GZ_ERR_BAD_ARG;
+}
+
+int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung, int variant, int num_cus,
+            int lds_per_cu, gz_plan_t* plan) {
+  return plan_impl(types, M, N, K, layoutA, layoutB, rung, variant, num_cus, lds_per_cu, ~(size_t)0, plan);
+}
+
+int gz_plan_static_scratch(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, int rung, int variant,
+                           int num_cus, int lds_per_cu, gz_plan_t* plan) {
+  return plan_impl(types, M, N, K, layoutA, layoutB, rung, variant, num_cus, lds_per_cu,
+                   (size_t)GZ_STATIC_SCRATCH_BYTES, plan);
 }
 
 const char* gz_rung_name(int rung) { return (rung >= 0 && rung < GZ_NUM_RUNGS) ? kRungNames[rung] : "auto"; }

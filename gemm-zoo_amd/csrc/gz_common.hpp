@@ -295,6 +295,9 @@ int current_device_index();
 // (one buffer per device and stream, grown with hipMalloc when a call needs more), or - inside the entry point that
 // allocates nothing - the static buffer, which refuses what it cannot hold.  Returns a gz_status.
 int workspace_acquire(size_t bytes, hipStream_t s, void** out);
+// The most workspace_acquire can give on the calling thread right now: unbounded from the pool, the size of the static
+// buffer inside the entry point that allocates nothing.  The launcher's own choice stays within it.
+size_t workspace_limit();
 
 // Raises a kernel's dynamic LDS limit once per device instead of on every launch.
 #define GZ_SET_LDS_LIMIT(kern, bytes)                                                                        \

@@ -3,7 +3,6 @@
 
 #include <stddef.h>
 #include <stdint.h>
-#include <stdlib.h>
 
 #include "../../include/gemm_zoo.h"
 
@@ -13,10 +12,10 @@ struct MfmaCfg {
   int id;       // variant id (1-based; 0 means "let the launcher choose")
   int bm, bn;   // work-group tile
   int waves_m, waves_n;
-  int hand_scheduled;  // fast path: 0 compiler-scheduled, 1 fixed sequence / two 128-byte buffers,
-                       // 2 fixed sequence / four 64-byte buffers or a ring of five (32x32 matrix instructions),
-                       // 3 as 2 with the 16x16 matrix instructions where a kernel with them exists,
-                       // 4 as 3, and the tiles past the last whole round of the compute units cut along K
+  int ring;     // 0: the compiler-scheduled kernels (register-staged, or direct-to-LDS where one exists for the tile);
+                // 1: the hand-scheduled ring kernel wherever the problem allows it, persistent past one round of
+                //    the compute units; 2: the same kernel with one work-group per tile
+  bool stream_k;  // the tiles past the last whole round of the compute units are cut along K (see mfma_plan_streamk)
 };
 
 // K slab per tile row is 128 bytes whatever the element type.
@@ -24,23 +23,26 @@ constexpr int MFMA_SLAB_BYTES = 128;
 constexpr int MFMA_LDS_PITCH = 144;
 
 static const MfmaCfg kMfmaCfgs[] = {
-    {1, 256, 256, 2, 2, 0},  // 4 waves of 128x128: fewest LDS bytes per MFMA
-    {2, 256, 256, 2, 4, 0},  // 8 waves of 128x64: two waves per SIMD hide each other's waits
-    {3, 128, 128, 2, 2, 0},  // small tile for small problems / ragged tails
-    {4, 256, 128, 2, 2, 0},  // 4 waves of 128x64
-    {5, 256, 256, 2, 2, 1},  // tile of variant 1 with the hand-scheduled main loop
-    {6, 256, 256, 2, 2, 2},  // tile of variant 1, hand-scheduled, four-buffer pipeline
-    {7, 256, 256, 2, 4, 2},  // tile of variant 2 (8 waves), hand-scheduled, four-buffer pipeline
-    {8, 256, 256, 2, 2, 3},  // tile of variant 1, hand-scheduled, ring of five buffers, 16x16 matrix instructions
-    {9, 256, 256, 2, 4, 3},  // tile of variant 2 (8 waves), the same
-    {10, 256, 256, 2, 2, 4},  // variant 8 with the stream-K decomposition wherever it applies (see mfma_plan_streamk)
-    {11, 256, 256, 2, 4, 4},  // variant 9, the same
+    {1, 256, 256, 2, 2, 0, false},   // 4 waves of 128x128: fewest LDS bytes per MFMA
+    {2, 256, 256, 2, 4, 0, false},   // 8 waves of 128x64: two waves per SIMD hide each other's waits
+    {3, 128, 128, 2, 2, 0, false},   // small tile for small problems / ragged tails
+    {4, 256, 128, 2, 2, 0, false},   // 4 waves of 128x64
+    {5, 256, 256, 2, 2, 1, false},   // tile of variant 1, hand-scheduled: ring of five buffers, 16x16 matrix instructions
+    {6, 256, 256, 2, 4, 1, false},   // tile of variant 2 (8 waves), the same
+    {7, 256, 256, 2, 2, 1, true},    // variant 5 with the stream-K decomposition wherever it applies
+    {8, 256, 256, 2, 4, 1, true},    // variant 6, the same
+    {9, 256, 256, 2, 2, 2, false},   // variant 5 with one work-group per tile (for comparisons with the persistent launch)
+    {10, 256, 256, 2, 4, 2, false},  // variant 6, the same
 };
 constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
+// positions in the table
+enum { MFMA_CFG_256_W4 = 0, MFMA_CFG_256_W8 = 1, MFMA_CFG_128 = 2, MFMA_CFG_256x128 = 3, MFMA_CFG_RING_W4 = 4,
+       MFMA_CFG_RING_W8 = 5 };
+enum { MFMA_VARIANT_RING_W4 = 5, MFMA_VARIANT_RING_W8 = 6, MFMA_VARIANT_STREAMK_W4 = 7, MFMA_VARIANT_STREAMK_W8 = 8 };
 
-// the most any kernel of the configuration asks for: the deep-pipeline kernels keep up to five buffers of 64-byte rows
+// the most any kernel of the configuration asks for: the ring kernel keeps five buffers of half a slab each
 inline int mfma_lds_bytes(const MfmaCfg& c) {
-  return c.hand_scheduled >= 2 ? 5 * (c.bm + c.bn) * 64 : 2 * (c.bm + c.bn) * MFMA_LDS_PITCH;
+  return c.ring ? 5 * (c.bm + c.bn) * 64 : 2 * (c.bm + c.bn) * MFMA_LDS_PITCH;
 }
 
 // How a problem sits on a tile configuration (16-byte alignment of the pointers is the caller's to check):
@@ -109,10 +111,11 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   if (num_cus <= 0) num_cus = 256;
   const int in_size = mfma_in_size(types);
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
-  // candidates: 256x256 (id 6), 256x128 (id 4), 128x128 (id 3)
-  const int cand[3] = {5, 3, 2};
+  // candidates: 256x256 (on the ring kernel where the types and the layout of A allow it), 256x128, 128x128
+  const bool ring_ok = a_rows && types != GZ_F32F32F32;
+  const int cand[3] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128, MFMA_CFG_128};
   double best = 0;
-  int pick = 5;
+  int pick = cand[0];
   for (int i = 0; i < 3; i++) {
     const MfmaCfg& c = kMfmaCfgs[cand[i]];
     const long long tiles = (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
@@ -160,50 +163,43 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     }
   }
   *out = kMfmaCfgs[pick];
-  if (pick == 5 && (types == GZ_BF16BF16BF16 || types == GZ_F16F16F16) && a_rows && b_cols) {
-    // 16-bit output, K-contiguous B: eight waves while the grid is small, and at every size on whole tiles (their
-    // epilogue is bound by the number of its stores; 4096^3 with operands rotating through seven sets, us, four /
-    // eight waves: bf16 -> bf16 103.5 / 101.7, fp16 110.5 / 106.6).  With an fp32 output four waves: level at 4096^3
-    // (105.2 / 105.4) and ahead beyond (4096^2 x 8192 194.5 / 197.8, 8192^3 770.6 / 790.8); they are also the less
-    // sensitive to operands that come from HBM rather than from the last-level cache (three sets / seven sets:
-    // 101.2 / 103.7 against 99.7 / 106.9 for eight waves).
+  if (pick == MFMA_CFG_RING_W4) {
+    // Waves per 256 x 256 tile on the ring kernel.
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
-    if (tiles <= 2LL * num_cus || (M % 256 == 0 && N % 256 == 0)) *out = kMfmaCfgs[6];
-  }
-  // 8-bit floats on the four-buffer kernel (column-major A never gets here: mfma_adjust_general), K-contiguous B: eight waves
-  if (pick == 5 && (types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) && a_rows && b_cols) *out = kMfmaCfgs[6];
-  // 8-bit floats, row-major A: the whole-line ring with the 16x16x128 instruction; eight waves up to three rounds of
-  // tiles (their 16-bit epilogue has more stores in flight), four beyond.  e4m3, us, four / eight waves, row/row:
-  // 4096^3 56.2 / 53.3, 5120^3 122.8 / 115.7, 6144^3 221.5 / 213.0, 4096^2 x 8192 99.6 / 99.0, 8192^3 404.9 / 419.4;
-  // row/col 4096^3 53.8 / 50.9, 8192^3 386.5 / 401.4.
-  if (pick == 5 && (types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16) && a_rows) {
-    const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
-    *out = kMfmaCfgs[tiles >= 4LL * num_cus && b_cols ? 7 : 8];   // (a row-major B: eight waves at every size, see below)
-  }
-  // int8 and the 16-bit types, both operands K-contiguous: the same tile and waves on the kernel with the 16x16
-  // matrix instructions (ids 8 and 9), which spend less energy per product on a part that runs against its power
-  // limit.  Interleaved runs, us, 32x32 / 16x16 instructions (hipBLASLt on the same operands): bf16 -> f32 4096^3
-  // 107.1 / 99.0 (105.0), 4096^2 x 8192 202.5 / 198.9 (196.6), 8192^3 798 / 789 (789); bf16 -> bf16 4096^3 105.0 /
-  // 97.0 (89.7); fp16 112.2 / 101.9 (95.0); int8 8192^3 443.7 / 423.3 on four waves, 430.9 on eight (450.5).
-  if (a_rows && (types == GZ_S8S8S32 || in_size == 2)) {   // (either layout of B: a row-major one through transposing reads)
-    if (out->id == 6) *out = kMfmaCfgs[7];
-    else if (out->id == 7) *out = kMfmaCfgs[8];
-    // Four waves are for grids of whole rounds.  Where compute units stay empty, or in the last of a few rounds,
-    // the busy ones have more of the chip's power and of their L2 to themselves, and eight waves use that better
-    // (two waves per SIMD cover each other's waits).  us, four / eight waves, K = 512, 1024, 4096 -
-    // bf16 -> f32: 3072^2 (144 tiles) 21.6 / 18.6, 29.9 / 26.4, 81.3 / 73.9; 3584^2 (196) 22.8 / 22.6, 32.2 / 31.4,
-    // 85.8 / 83.3; 4096^2 (256) 24.1 / 25.0, 34.9 / 35.3, 98.0 / 98.6; 4608^2 (324) 44.3 / 38.3, 63.3 / 56.9,
-    // 178.1 / 170.3; 5120^2 (400) 45.3 / 39.6, 66.5 / 59.6, 184.1 / 181.5; 6144^2 (576) 67.8 / 60.5, 96.1 / 89.4,
-    // 274.8 / 273.9; int8 the same way (3072^2 15.8 / 14.2, 20.4 / 18.6, 46.2 / 42.4; 5120^2 34.9 / 30.3,
-    // 44.6 / 39.5, 106.6 / 99.0).  From three rounds on four waves: 8192^3 770.6 / 790.8.
-    // A row-major B comes out of LDS through the transposing reads, two per fragment: eight waves at every size
-    // (us, four / eight waves, row/row: bf16 4096^3 104.5 / 101.3, 8192^3 823.5 / 791.5, 4096^2 x 1024 39.0 / 37.5,
-    // 4000^2 x 4096 109.3 / 102.6; fp16 4096^3 111.3 / 104.8, 8192^3 856 / 810; int8 4096^3 61.9 / 59.6, 8192^3
-    // 444.2 / 437.6, 8000^2 x 8192 448.2 / 435.1; e4m3 8192^3 400.8 / 394.7, 8000^2 x 8192 431.8 / 409.6).
-    if (out->id == 8) {
-      const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
-      if (!b_cols || (tiles % num_cus != 0 && tiles / num_cus < 3)) *out = kMfmaCfgs[8];
+    const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
+    bool eight = false;
+    if (f8) {
+      // 8-bit floats: eight waves up to three rounds of tiles (their 16-bit epilogue has more stores in flight),
+      // four beyond.  e4m3, us, four / eight waves, row/row: 4096^3 56.2 / 53.3, 5120^3 122.8 / 115.7, 6144^3
+      // 221.5 / 213.0, 4096^2 x 8192 99.6 / 99.0, 8192^3 404.9 / 419.4; row/col 4096^3 53.8 / 50.9, 8192^3
+      // 386.5 / 401.4.  (A row-major B: eight waves at every size, see below.)
+      eight = !(tiles >= 4LL * num_cus && b_cols);
+    } else {
+      // 16-bit output, K-contiguous B: eight waves while the grid is small, and at every size on whole tiles (their
+      // epilogue is bound by the number of its stores; 4096^3 with operands rotating through seven sets, us, four /
+      // eight waves: bf16 -> bf16 103.5 / 101.7, fp16 110.5 / 106.6).  With an fp32 output four waves: level at
+      // 4096^3 (105.2 / 105.4) and ahead beyond (4096^2 x 8192 194.5 / 197.8, 8192^3 770.6 / 790.8); they are also
+      // the less sensitive to operands that come from HBM rather than from the last-level cache (three sets / seven
+      // sets: 101.2 / 103.7 against 99.7 / 106.9 for eight waves).
+      if ((types == GZ_BF16BF16BF16 || types == GZ_F16F16F16) && b_cols &&
+          (tiles <= 2LL * num_cus || (M % 256 == 0 && N % 256 == 0)))
+        eight = true;
+      // Four waves are for grids of whole rounds.  Where compute units stay empty, or in the last of a few rounds,
+      // the busy ones have more of the chip's power and of their L2 to themselves, and eight waves use that better
+      // (two waves per SIMD cover each other's waits).  us, four / eight waves, K = 512, 1024, 4096 -
+      // bf16 -> f32: 3072^2 (144 tiles) 21.6 / 18.6, 29.9 / 26.4, 81.3 / 73.9; 3584^2 (196) 22.8 / 22.6, 32.2 / 31.4,
+      // 85.8 / 83.3; 4096^2 (256) 24.1 / 25.0, 34.9 / 35.3, 98.0 / 98.6; 4608^2 (324) 44.3 / 38.3, 63.3 / 56.9,
+      // 178.1 / 170.3; 5120^2 (400) 45.3 / 39.6, 66.5 / 59.6, 184.1 / 181.5; 6144^2 (576) 67.8 / 60.5, 96.1 / 89.4,
+      // 274.8 / 273.9; int8 the same way (3072^2 15.8 / 14.2, 20.4 / 18.6, 46.2 / 42.4; 5120^2 34.9 / 30.3,
+      // 44.6 / 39.5, 106.6 / 99.0).  From three rounds on four waves: 8192^3 770.6 / 790.8.
+      if (tiles % num_cus != 0 && tiles / num_cus < 3) eight = true;
+      // A row-major B comes out of LDS through the transposing reads, two per fragment: eight waves at every size
+      // (us, four / eight waves, row/row: bf16 4096^3 104.5 / 101.3, 8192^3 823.5 / 791.5, 4096^2 x 1024 39.0 / 37.5,
+      // 4000^2 x 4096 109.3 / 102.6; fp16 4096^3 111.3 / 104.8, 8192^3 856 / 810; int8 4096^3 61.9 / 59.6, 8192^3
+      // 444.2 / 437.6, 8000^2 x 8192 448.2 / 435.1; e4m3 8192^3 400.8 / 394.7, 8000^2 x 8192 431.8 / 409.6).
+      if (!b_cols) eight = true;
     }
+    if (eight) *out = kMfmaCfgs[MFMA_CFG_RING_W8];
   }
   return best;
 }
@@ -229,8 +225,9 @@ inline void mfma_adjust_general(int types, int cls, int layoutA, MfmaCfg* c) {
   const bool staged = cls == MFMA_SHAPE_GENERAL || layoutA != GZ_ROW_MAJOR;
   if (!staged || c->bm != 256 || c->bn != 256) return;
   const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
-  if (f8) *c = kMfmaCfgs[0];
-  else if (types != GZ_F32F32F32) *c = kMfmaCfgs[1];
+  if (f8) *c = kMfmaCfgs[MFMA_CFG_256_W4];
+  else if (types != GZ_F32F32F32) *c = kMfmaCfgs[MFMA_CFG_256_W8];
+  else *c = kMfmaCfgs[MFMA_CFG_256_W4];
 }
 
 // Ragged last round.  When the 256x256 tiles of a problem fill some rounds of the compute units and then leave a
@@ -310,8 +307,8 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   if (direct_before && !direct_after) cost_main *= types == GZ_F32F32F32 ? 2.2 : mfma_in_size(types) == 2 ? 1.2 : 1.5;
   // on the register-staged kernel eight waves carry a 256 x 256 tile of 16-bit elements better than four
   // (fp16 4095 x 4097 x 1023, row-major B: 119 us against 158)
-  if (!direct_after && main_cfg.bm == 256 && main_cfg.bn == 256 && mfma_in_size(types) == 2) main_cfg = kMfmaCfgs[6];
-  tail_cfg = kMfmaCfgs[2];   // 128 x 128: the strip in as many work-groups as it has row blocks
+  if (!direct_after && main_cfg.bm == 256 && main_cfg.bn == 256 && mfma_in_size(types) == 2) main_cfg = kMfmaCfgs[MFMA_CFG_256_W8];
+  tail_cfg = kMfmaCfgs[MFMA_CFG_128];   // 128 x 128: the strip in as many work-groups as it has row blocks
   // What the cut-off columns cost depends on K, the rounds above do not say it: in us, the dot products
   // 3 + (M / 4096) (K bytes / 2048) (4 + 1.8 r) (one column of 4095 x 1023 fp16: 11 us; eight of 4096 x 4096: 75),
   // the same strip on 128 x 128 tiles 5 + 11.5 (M / 4096) (K bytes / 2048) (15-18 us at K = 1024, 44-52 at 4096),
@@ -352,11 +349,11 @@ inline int mfma_resolve_cut(int types, int M, int N, int K, int layoutA, int lay
 struct StreamKPlan {
   int dp_tiles, sk_tiles, blocks, q, rem;   // see struct StreamK of the kernel
   int slots;                                // workspace slots of 256 x 256 accumulators
-  MfmaCfg cfg;                              // tile configuration (id 8 or 9)
+  MfmaCfg cfg;                              // tile configuration (the ring kernel on four or eight waves)
   double estimate_us;
 };
 constexpr long long MFMA_STREAMK_SLOT_BYTES = 256ll * 256 * 4;
-// forced: an explicit stream-K variant (ids 10, 11): taken wherever it can run; otherwise only where the estimate says so
+// forced: an explicit stream-K variant: taken wherever it can run; otherwise only where the estimate says so
 inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, bool forced,
                               const MfmaCfg* forced_cfg, StreamKPlan* out) {
   if (num_cus <= 0) num_cus = 256;
@@ -364,10 +361,10 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
   if (!(types == GZ_S8S8S32 || in_size == 2) || layoutA != GZ_ROW_MAJOR || layoutB != GZ_COL_MAJOR) return false;
   MfmaCfg cfg;
   double single_rounds = mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, &cfg);
-  if (forced) cfg = kMfmaCfgs[forced_cfg->waves_n == 4 ? 8 : 7];
-  else if (cfg.id != 8 && cfg.id != 9) {
+  if (forced) cfg = kMfmaCfgs[forced_cfg->waves_n == 4 ? MFMA_CFG_RING_W8 : MFMA_CFG_RING_W4];
+  else if (cfg.id != MFMA_VARIANT_RING_W4 && cfg.id != MFMA_VARIANT_RING_W8) {
     // a smaller tile was preferred for the whole problem (few tiles): stream-K still competes, on the 256 x 256 tile
-    cfg = kMfmaCfgs[in_size == 2 ? 8 : 7];
+    cfg = kMfmaCfgs[in_size == 2 ? MFMA_CFG_RING_W8 : MFMA_CFG_RING_W4];
   }
   if (mfma_shape_class(cfg, in_size, M, N, K, layoutA, layoutB) == MFMA_SHAPE_GENERAL) return false;
   const int nslab = K / (MFMA_SLAB_BYTES / in_size);
@@ -429,14 +426,13 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
   return out->estimate_us < 0.95 * best * round_us;
 }
 
-// Work-groups of a launch of whole tiles on the ring kernel with the 16x16 instructions: past one round of the compute
-// units the kernel is persistent, one work-group per compute unit walking tiles b, b + grid, ... (the order in which
-// the hardware deals work-groups out anyway) and asking for its next tile's first slab before it stores the current
-// one.  GZ_MFMA_PERSISTENT=0 in the environment keeps one work-group per tile (for comparisons).
+// Work-groups of a launch of whole tiles on the ring kernel: past one round of the compute units the kernel is
+// persistent, one work-group per compute unit walking tiles b, b + grid, ... (the order in which the hardware deals
+// work-groups out anyway) and asking for its next tile's first slab before it stores the current one.  (Variants 9
+// and 10 launch one work-group per tile instead, for comparisons.)
 inline long long mfma_persistent_grid(long long tiles, int num_cus) {
-  static const bool on = [] { const char* e = getenv("GZ_MFMA_PERSISTENT"); return !(e && e[0] == '0'); }();
   if (num_cus <= 0) num_cus = 256;
-  return on && tiles > num_cus ? num_cus : tiles;
+  return tiles > num_cus ? num_cus : tiles;
 }
 
 // Shape class of a launch: the direct-to-LDS kernels also need 16-byte aligned operands.

@@ -10,15 +10,16 @@
 // ends up with 4 consecutive columns of one output row and the epilogue stores
 // are 128-bit (fp32 / int32) or 64-bit (16-bit outputs).
 //
-// Three kernels share that tiling:
-//   mfma_gemm_kernel  general: any layout, any shape (predicated EDGE instantiation), any alignment.
-//                     Slabs are staged global -> registers -> LDS ([row][k], pitch 144 B: the 16-byte pad
-//                     makes the fragment reads of 16 consecutive rows hit 16 distinct 4-bank groups);
-//                     operands whose contiguous dimension is not K (row-major B, column-major A) are
-//                     transposed in registers on the way in.
-//   mfma_dtl_kernel   fast path for K-contiguous operands, whole tiles, 16-byte alignment: slabs go
-//                     global -> LDS directly (global_load_lds_dwordx4), unpadded swizzled rows.
-//   mfma_asm_kernel   the same data movement with a hand-placed instruction sequence (variant 5).
+// The kernels of the rung:
+//   mfma_gemm_kernel   general: any layout, any shape (predicated EDGE instantiation), any alignment.
+//                      Slabs are staged global -> registers -> LDS ([row][k], pitch 144 B: the 16-byte pad
+//                      makes the fragment reads of 16 consecutive rows hit 16 distinct 4-bank groups);
+//                      operands whose contiguous dimension is not K (row-major B, column-major A) are
+//                      transposed in registers on the way in.
+//   mfma_dtl_kernel    compiler-scheduled fast path for whole tiles with 16-byte aligned rows: slabs go
+//                      global -> LDS directly (global_load_lds_dwordx4), unpadded swizzled rows.
+//   mfma_ring16_kernel (rung4_mfma_ring16.hpp) the hand-scheduled 256 x 256 kernel with the 16x16 matrix
+//                      instructions and a ring of five LDS buffers: what the launcher runs on big problems.
 //
 // Stands in for nvidia/kernels/sm_80/{bf16,fp16}_mma_gemm.cuh and
 // intel/kernels/xe_gemm_*_m8k16.hpp (same operation, new design).
@@ -956,23 +957,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 }
 
 // ---------------------------------------------------------------------------
-// Hand-scheduled fast path.
-//
-// Same data movement as mfma_dtl_kernel (direct-to-LDS copies, swizzled unpadded rows, two LDS buffers, one
-// barrier per slab), but the main loop is a fixed instruction sequence: a wavefront issues in order, so one
-// memory instruction is placed after each MFMA and nowhere else.  Measured on MI355X, 16 MFMAs with 8
-// ds_read_b128 and 4 LDS copies slotted in this way run at the rate of 16 bare MFMAs, while the same
-// instructions bunched together (the compiler's order) cost 40-50 % more.  The sequence is written as
-// volatile asm statements so that neither the scheduler nor the wait-count pass (which, with an LDS copy
-// pending, waits for lgkmcnt(0) before the first MFMA of every step) can change it; all s_waitcnt are
-// placed by hand:
-//   step start : lgkmcnt(0)  - the fragments of this step were requested one step (>= 8 MFMAs) ago
-//   barrier    : vmcnt(0) lgkmcnt(0) - this wave's copies of the next slab have landed, its reads of the
-//                current buffer have returned
-// Per slab (4 steps): step 0..2 read the next step's fragments from the current buffer, step 3 (after the
-// barrier) reads step 0 of the next slab from the other buffer.  The copies of slab kt+2 into the buffer
-// freed by that barrier are issued in step 3 of slab kt and step 0 of slab kt+1, so they have two more
-// steps to land.
+// Pieces of the hand-scheduled kernel (rung4_mfma_ring16.hpp).  Its main loop is a fixed instruction sequence
+// written as volatile asm statements, so that neither the scheduler nor the wait-count pass (which, with an LDS copy
+// pending, waits for lgkmcnt(0) before the first MFMA of every step) can change it; every s_waitcnt is placed by hand.
 // ---------------------------------------------------------------------------
 template <int OFF> __device__ __forceinline__ void asm_ds_read16(u32x4_t& dst, uint32_t addr) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
@@ -984,231 +971,29 @@ __device__ __forceinline__ void asm_set_m0(uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory");
 }
 // 64 lanes x 16 bytes from sbase + voff + OFF (per lane) to LDS at M0 + OFF + 16 * lane: the immediate offset
-// applies to both addresses, so the caller passes the source base minus OFF.
-template <int OFF> __device__ __forceinline__ void asm_copy16(uint32_t voff, const void* sbase_minus_off) {
+// applies to both addresses, so the caller takes OFF off the source address again (in sbase or in voff).
+template <int OFF> __device__ __forceinline__ void asm_copy16(uint32_t voff, const void* sbase) {
   static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
-  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase_minus_off), "i"(OFF) : "memory");
+  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase), "i"(OFF) : "memory");
 }
-template <int TYPES>
-__device__ __forceinline__ void asm_mfma32(typename AccVec<TYPES>::type& c, const u32x4_t& first, const u32x4_t& second) {
-  if constexpr (TYPES == GZ_S8S8S32)
-    asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
-  else if constexpr (TYPES == GZ_F16F16F16)
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
-  else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
+// The same under a lane mask (a scalar register pair): an all-zero mask turns the instruction into a no-op that
+// still takes its place in the sequence and in the vmcnt order.
+template <int OFF> __device__ __forceinline__ void asm_copy16_masked(uint32_t voff, const void* sbase, uint64_t mask) {
+  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
+  asm volatile("s_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2\n\ts_mov_b64 exec, -1"
+               :
+               : "v"(voff), "s"(sbase), "i"(OFF), "s"(mask)
+               : "memory");
 }
-
-// v_mfma_f32_32x32x64_f8f6f4 on 8-bit floats: 32 bytes per lane and operand, given as the fragments of two
-// consecutive 32-byte K steps (cbsz / blgp select the format of the two operands: 0 e4m3, 1 e5m2)
 typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
-template <int TYPES>
-__device__ __forceinline__ void asm_mfma_f8(typename AccVec<TYPES>::type& c, const u32x4_t& first0, const u32x4_t& first1,
-                                            const u32x4_t& second0, const u32x4_t& second1) {
-  const u32x8_t f = __builtin_shufflevector(first0, first1, 0, 1, 2, 3, 4, 5, 6, 7);
-  const u32x8_t s = __builtin_shufflevector(second0, second1, 0, 1, 2, 3, 4, 5, 6, 7);
-  if constexpr (TYPES == GZ_E5M2E5M2F16)
-    asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(c) : "v"(f), "v"(s));
-  else
-    asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(f), "v"(s));
-}
-
-// orders later reads of an accumulator after every asm statement that precedes this one
-template <int TYPES> __device__ __forceinline__ void asm_touch_acc(typename AccVec<TYPES>::type& c) {
-  asm volatile("" : "+a"(c));
-}
-
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
-__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
-    mfma_asm_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
-  using T = Traits<TYPES>;
-  using in_t = typename T::in_t;
-  using out_t = typename T::out_t;
-  using acc_v = typename AccVec<TYPES>::type;
-  constexpr int NW = WAVES_M * WAVES_N;
-  constexpr int ES = (int)sizeof(in_t);
-  constexpr int EPV = 16 / ES;
-  constexpr int BK = SLAB_BYTES / ES;
-  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  constexpr int FM = WM / 32, FN = WN / 32;
-  constexpr int ROWB = SLAB_BYTES;
-  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
-  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int A_PW = BM / 8 / NW, B_PW = BN / 8 / NW;
-  constexpr int NCP = A_PW + B_PW, NMMA = FM * FN, NRD = FM + FN;
-  static_assert(A_PW <= 8 && B_PW <= 8 && A_PW % 2 == 0 && B_PW % 2 == 0, "a copy group must fit the immediate offset range");
-  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must divide over the waves");
-  static_assert(KSTEPS == 4, "the step schedule below is written for four MFMA steps per slab");
-
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-  int tm, tn;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int K = g.K;
-
-  // ---- copy addressing (see mfma_dtl_kernel) ----
-  const int lr = lane >> 3, lp = lane & 7;
-  uint32_t a_voff[2], b_voff[2];
-#pragma unroll
-  for (int par = 0; par < 2; par++) {
-    const int ca = lp ^ lr ^ (((wave * A_PW) & 1) ^ par);
-    const int cb = lp ^ lr ^ (((wave * B_PW) & 1) ^ par);
-    a_voff[par] = (uint32_t)((lr * K + ca * EPV) * ES);
-    b_voff[par] = (uint32_t)((lr * K + cb * EPV) * ES);
-  }
-  const char* a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(m0 + 8 * wave * A_PW) * K * ES;
-  const char* b_ubase = reinterpret_cast<const char*>(g.B) + (size_t)(n0 + 8 * wave * B_PW) * K * ES;
-  const size_t group_step = (size_t)8 * K * ES;
-  // copy number C of the slab that starts at K byte `kbyte`: copies [0, A_PW) move this wave's A rows, the rest
-  // its B rows.  Each group has one M0 (set by copy_group_begin) in the middle of its LDS span.
-  auto copy_group_begin = [&](auto c_c, int st) {
-    constexpr int C = decltype(c_c)::value;
-    if constexpr (C == 0) asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024);
-    else if constexpr (C == A_PW) asm_set_m0(lds_base + st * STAGE_BYTES + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024);
-  };
-  auto copy_one = [&](auto c_c, int st, size_t kbyte) {
-    constexpr int C = decltype(c_c)::value;
-    copy_group_begin(c_c, st);
-    if constexpr (C < A_PW) {
-      constexpr int OFF = (C - A_PW / 2) * 1024;
-      asm_copy16<OFF>(a_voff[C & 1], a_ubase + C * group_step + kbyte - OFF);
-    } else {
-      constexpr int Tn = C - A_PW;
-      constexpr int OFF = (Tn - B_PW / 2) * 1024;
-      asm_copy16<OFF>(b_voff[Tn & 1], b_ubase + Tn * group_step + kbyte - OFF);
-    }
-  };
-
-  // ---- fragment addressing ----
-  const int frag_row = lane & 31, half = lane >> 5;
-  const int sw = dtl_swz(frag_row);
-  uint32_t a_addr[2][KSTEPS], b_addr[2][KSTEPS];
-#pragma unroll
-  for (int st = 0; st < 2; st++)
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-      const int pos = ((ks * 2 + half) ^ sw) * 16;
-      a_addr[st][ks] = lds_base + st * STAGE_BYTES + (wm * WM + frag_row) * ROWB + pos;
-      b_addr[st][ks] = lds_base + st * STAGE_BYTES + A_BYTES + (wn * WN + frag_row) * ROWB + pos;
-    }
-
-  acc_v acc[FM][FN];
-#pragma unroll
-  for (int i = 0; i < FM; i++)
-#pragma unroll
-    for (int j = 0; j < FN; j++)
-#pragma unroll
-      for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
-  // the zeroing above is ordinary code: pin it before the asm sequence (and give the VALU writes their wait
-  // states before an MFMA may read the accumulators)
-  static_for<NMMA>([&](auto q_c) {
-    constexpr int Q = decltype(q_c)::value;
-    asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
-  });
-  asm volatile("s_nop 7" ::: "memory");
-  u32x4_t af[2][FM], bf[2][FN];
-
-  // fragment read number R (A fragments first) of K step `ks` of buffer `st` into register set SET
-  auto read_one = [&](auto set_c, auto r_c, int st, int ks) {
-    constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value;
-    if constexpr (R < FM) asm_ds_read16<R * 32 * ROWB>(af[SET][R], a_addr[st][ks]);
-    else asm_ds_read16<(R - FM) * 32 * ROWB>(bf[SET][R - FM], b_addr[st][ks]);
-  };
-
-  // One MFMA step.  P: step within the slab; CUR: buffer of the slab.  The fragments of the next step are always
-  // requested (past the last slab they are stale data that nobody multiplies); `copy` says whether this step's
-  // quarter of the LDS copies is issued - a uniform run-time branch around a copy does not disturb the
-  // sequence, and one code path for every slab keeps the accumulators in the same registers throughout.
-  auto step = [&](auto p_c, auto cur_c, bool copy, int kt) {
-    constexpr int P = decltype(p_c)::value, CUR = decltype(cur_c)::value;
-    constexpr int SET = P & 1;
-    constexpr int RST = P < 3 ? CUR : (CUR ^ 1), RKS = P < 3 ? P + 1 : 0;
-    // copies: step 3 -> first quarter of slab kt+2 into CUR ; steps 0, 1, 2 -> the other quarters of slab kt+1
-    // into CUR^1 (the texture path needs most of a slab's time to move a slab, so the copies are spread evenly)
-    constexpr int QN = (P + 1) & 3;  // quarter number: step 3 -> 0, step 0 -> 1, step 1 -> 2, step 2 -> 3
-    constexpr int CB = QN * NCP / 4, CE = (QN + 1) * NCP / 4;
-    constexpr int NC = CE - CB;
-    constexpr int NOPS = NRD + NC;
-    const int cst = P == 3 ? CUR : (CUR ^ 1);
-    const size_t kbyte = (size_t)(kt + (P == 3 ? 2 : 1)) * SLAB_BYTES;
-    asm volatile("s_waitcnt lgkmcnt(0)");
-    static_for<NMMA>([&](auto q_c) {
-      constexpr int Q = decltype(q_c)::value;
-      asm_mfma32<TYPES>(acc[Q / FN][Q % FN], bf[SET][Q % FN], af[SET][Q / FN]);
-      static_for<NOPS>([&](auto o_c) {
-        constexpr int O = decltype(o_c)::value;
-        constexpr int SLOT = NOPS <= NMMA ? O : (O * NMMA) / NOPS;
-        if constexpr (SLOT == Q) {
-          if constexpr (O < NRD) {
-            read_one(std::integral_constant<int, SET ^ 1>{}, o_c, RST, RKS);
-          } else {
-            if (copy) copy_one(std::integral_constant<int, CB + O - NRD>{}, cst, kbyte);
-          }
-        }
-      });
-    });
-  };
-
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I3 = std::integral_constant<int, 3>;
-
-  // One slab: steps 0..2 from buffer CUR, barrier, step 3.
-  //   steps 0..2 issue quarters 1..3 of the copies of slab kt+1 (slab 1 was copied whole by the prologue)
-  //   step 3 issues quarter 0 of the copies of slab kt+2
-  auto slab = [&](auto cur_c, int kt, int ktiles) {
-    const bool later = kt >= 1 && kt + 1 < ktiles, first = kt + 2 < ktiles;
-    step(I0{}, cur_c, later, kt);
-    step(I1{}, cur_c, later, kt);
-    step(I2{}, cur_c, later, kt);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    step(I3{}, cur_c, first, kt);
-  };
-
-  const int ktiles = K / BK;  // >= 1 on this path
-  // Prologue: slab 0 and slab 1 copied whole; fragments of (slab 0, step 0) requested.
-  static_for<NCP>([&](auto c) { copy_one(c, 0, 0); });
-  if (ktiles > 1) static_for<NCP>([&](auto c) { copy_one(c, 1, (size_t)SLAB_BYTES); });
-  if (ktiles > 1) {
-    if constexpr (NCP == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if constexpr (NCP == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
-  asm volatile("s_barrier" ::: "memory");
-  static_for<NRD>([&](auto r) { read_one(I0{}, r, 0, 0); });
-
-  // Two slabs per trip so that the buffer index is a compile-time constant; the second one is skipped (not
-  // duplicated) when K has an odd number of slabs.
-  for (int kt = 0; kt < ktiles; kt += 2) {
-    slab(I0{}, kt, ktiles);
-    if (kt + 1 < ktiles) slab(I1{}, kt + 1, ktiles);
-  }
-  // The last MFMAs must have written their accumulators before ordinary code reads them: the hazard
-  // recogniser does not look inside asm statements, so the wait states are spelled out, and every
-  // accumulator is passed through an (empty) asm placed after them so that no read can be hoisted above.
-  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7" ::: "memory");
-  static_for<NMMA>([&](auto q_c) {
-    constexpr int Q = decltype(q_c)::value;
-    asm_touch_acc<TYPES>(acc[Q / FN][Q % FN]);
-  });
-
-  store_accumulators<TYPES, FM, FN>(g, acc, m0 + wm * WM, n0 + wn * WN, lane);
+// half a fragment of a row-major B through the transposing LDS reads
+template <int ES, int OFF> __device__ __forceinline__ void asm_ds_read_tr(u32x2_t& dst, uint32_t addr) {
+  if constexpr (ES == 2) asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
+  else asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(OFF));
 }
 
 }  // namespace gz
 
-#include "rung4_mfma_pipe4.hpp"
-#include "rung4_mfma_ring5.hpp"
 #include "rung4_mfma_ring16.hpp"
 
 namespace gz {
@@ -1217,7 +1002,7 @@ namespace gz {
 // Launcher
 // ---------------------------------------------------------------------------
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
-static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_scheduled, hipStream_t s) {
+static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipStream_t s) {
   const int tiles_m = ceil_div(g.M, BM), tiles_n = ceil_div(g.N, BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(WAVES_M * WAVES_N * 64);
   const size_t lds = 2u * (size_t)(BM + BN) * PITCH;
@@ -1244,39 +1029,27 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
 #define GZ_KERN(...) __VA_ARGS__   // a template-id with commas as one macro argument
 
   // The direct-to-LDS kernels: row-major A, whole K slabs, 16-byte aligned rows (the shape class says so), whole
-  // tiles or, on the hand-scheduled 256 x 256 kernels, any M and N (rows clamped).  hand_scheduled: 3 the ring of
-  // five buffers with the 16x16 instructions, 2 the older ring (32x32 instructions; not for the 8-bit floats) or
-  // the four-buffer kernel, 1 the two-buffer hand-scheduled kernel, 0 the compiler-scheduled ones.  fp32 runs the
-  // register-staged kernel only: its MFMAs are 8x longer per byte.
+  // tiles or, on the hand-scheduled 256 x 256 kernel, any M and N (rows clamped).  ring: 0 the compiler-scheduled
+  // kernels, 1 the hand-scheduled ring kernel with one work-group per compute unit walking the tiles of a grid of
+  // more than one round, 2 the same kernel with one work-group per tile.  fp32 runs the register-staged kernel only:
+  // its MFMAs are 8x longer per byte.
   constexpr bool TILE_256 = BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4);
-  constexpr bool F8 = is_fp8(TYPES);
-  const size_t ring_lds = 5u * (size_t)(BM + BN) * 64, pipe_lds = 4u * (size_t)(BM + BN) * 64;
+  const size_t ring_lds = 5u * (size_t)(BM + BN) * 64;
   const size_t dtl_lds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
-  const bool whole_lines = ((size_t)g.K * sizeof(typename Traits<TYPES>::in_t)) % 128 == 0;
-  // whole tiles on the ring kernel: one work-group per compute unit walks the tiles (mfma_persistent_grid)
-  const dim3 pgrid((unsigned)mfma_persistent_grid((long long)tiles_m * tiles_n, device_compute_units()));
+  const dim3 pgrid((unsigned)(ring == 1 ? mfma_persistent_grid((long long)tiles_m * tiles_n, device_compute_units())
+                                        : (long long)tiles_m * tiles_n));
   if constexpr (TYPES != GZ_F32F32F32) {
     if constexpr (TILE_256) {
-      if (shape_class == MFMA_SHAPE_RAGGED_MN && akc && hand_scheduled >= 2) {
-        if (hand_scheduled == 3) {
-          if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
-          else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
-        }
-        if constexpr (!F8)
-          if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring5_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>), ring_lds);
-        if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, true>), pipe_lds);
-        if constexpr (WAVES_N == 2) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, true>), pipe_lds);
+      if (ring && akc && shape_class == MFMA_SHAPE_RAGGED_MN) {
+        if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
+        else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
+      }
+      if (ring && akc && !edge) {
+        if (bkc) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});
+        else GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
       }
     }
     if (!edge && akc && bkc) {  // whole tiles, both operands K-contiguous
-      if constexpr (TILE_256) {
-        if (hand_scheduled == 3 && whole_lines) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});
-        if constexpr (!F8)
-          if (hand_scheduled >= 2 && whole_lines) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring5_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds);
-        if (hand_scheduled >= 2) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), pipe_lds);
-      }
-      if constexpr (!F8 && BM == 256 && BN == 256 && WAVES_M == 2 && WAVES_N == 2)
-        if (hand_scheduled == 1) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_asm_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), dtl_lds);
       // The compiler-scheduled direct-to-LDS kernel is kept for the eight-wave 256x256 tile only: with four waves the
       // register-staged kernel below, whose loads and LDS stores are spread between the MFMAs, measured faster on
       // every tile (interleaved runs, us, direct / register-staged: bf16 2048^3 128x128 28.6 / 27.1, 256x128 39.2 /
@@ -1284,15 +1057,8 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int hand_schedu
       if constexpr (WAVES_M * WAVES_N == 8) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), dtl_lds);
     }
     if (!edge && akc && !bkc) {  // whole tiles, row-major A and B: direct-to-LDS copies, transposing LDS reads for B
-      // (128x128 and 256x256 only: on 256x128 the register-staged kernel is faster, 2048^3 50.0 / 43.0 us, 4096^3 185 / 150)
+      // (128x128 only: on 256x128 the register-staged kernel is faster, 2048^3 50.0 / 43.0 us, 4096^3 185 / 150)
       if constexpr (BM == 128 && BN == 128) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_dtl_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>), dtl_lds);
-      if constexpr (TILE_256)
-        if (hand_scheduled == 3 && whole_lines) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
-      if constexpr (TILE_256 && WAVES_N == 2) {
-        if constexpr (!F8)
-          if (hand_scheduled >= 2 && whole_lines) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring5_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>), ring_lds);
-        if (hand_scheduled >= 2) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_pipe4_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false>), pipe_lds);
-      }
     }
   }
 #undef GZ_LAUNCH_DIRECT
@@ -1524,11 +1290,10 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
     case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);
     case 3: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 0, s);
     case 4: return launch_cfg<TYPES, 256, 128, 2, 2>(g, edge, 0, s);
-    case 5: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 1, s);
-    case 6: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s);
-    case 7: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s);
-    case 8: case 10: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 3, s);
-    case 9: case 11: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 3, s);
+    case 5: case 7: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 1, s);
+    case 6: case 8: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 1, s);
+    case 9: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s);
+    case 10: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s);
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);
@@ -1571,10 +1336,13 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
   GemmArgs<TYPES> g = args;
   const int num_cus = device_compute_units();
   g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), num_cus);
-  if ((variant == 0 || variant == 10 || variant == 11) && g.K > 0 && g.ldd == g.N) {
+  if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && g.K > 0 && g.ldd == g.N) {
     StreamKPlan skp;
     const MfmaCfg* forced = variant == 0 ? nullptr : &kMfmaCfgs[variant - 1];
-    if (mfma_plan_streamk(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, num_cus, forced != nullptr, forced, &skp)) {
+    // the launcher's own choice stays within the workspace this entry point may use (the entry point that
+    // allocates nothing has a fixed one); an explicit stream-K variant is refused by workspace_acquire instead
+    if (mfma_plan_streamk(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, num_cus, forced != nullptr, forced, &skp) &&
+        (forced || (size_t)skp.slots * MFMA_STREAMK_SLOT_BYTES <= workspace_limit())) {
       const int cls = mfma_launch_class(skp.cfg, (int)sizeof(typename Traits<TYPES>::in_t), g.M, g.N, g.K, g.layoutA,
                                         g.layoutB, g.A, g.B, g.C, g.D);
       if (cls != MFMA_SHAPE_GENERAL) {   // (unaligned operands: the plain launch below, on the register-staged kernel)

@@ -198,74 +198,82 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   const int nc = 2 * nslab_seg;  // copy groups
   const size_t k_byte0 = (size_t)slab0 * LINE;   // first K byte of this run within a row
 
-  // ---- copy addressing (as mfma_ring5_kernel): lane -> (row ci of the 8 rows of a copy, LDS slot cs) ----
+  // ---- copy addressing: lane -> (row ci of the 8 rows of a copy, LDS slot cs) ----
+  // A copy is ONE instruction of the main loop, with nothing scalar around it.  Its source address has three parts:
+  // a scalar base that every copy of the operand in a K step shares (the tile's first row at the K offset of the
+  // slab that is being fetched; a_cp / b_cp below, advanced once per slab or K step), a per-lane offset kept in a
+  // register per (parity, copy of the group) and computed once per tile - which 16 rows, which parity, the lane's
+  // row and piece - and the immediate.  The immediate also moves the LDS address (that is what it is for: the copies
+  // of a group step through LDS with it, under one M0), so it is taken off the per-lane offset again; COPY_BIAS keeps
+  // that difference non-negative and is taken off the scalar base.  (Before: one scalar base per copy, computed in
+  // the loop with four to six scalar instructions, and a lane mask around every copy for the groups past the end of
+  // K - seven to ten instructions per copy between two MFMAs, where a wave that is alone on its SIMD issues one
+  // instruction every four cycles and an MFMA leaves room for three.)
+  constexpr uint32_t COPY_BIAS = 4096;
   const int ci = lane >> 3, cs = lane & 7;
-  const uint32_t voff[2] = {(uint32_t)(ci * K * ES + ((cs ^ ci) * 16)), (uint32_t)(ci * K * ES + ((cs ^ ci ^ 1) * 16))};
-  const size_t group_step = (size_t)16 * K * ES, parity_step = (size_t)8 * K * ES;
-  const char* a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(m0 + 16 * wave * A_PW) * K * ES + k_byte0;
-  auto b_base_of = [&](int n_first) -> const char* {   // first byte this wave copies of the B rows or columns from n_first on
-    if constexpr (B_KC) return reinterpret_cast<const char*>(g.B) + (size_t)(n_first + 16 * wave * B_PW) * K * ES + k_byte0;
-    else return reinterpret_cast<const char*>(g.B) + ((size_t)(wave * B_PW * (1024 / (BN * ES))) * g.N + n_first) * ES;
-  };
+  const int N = g.N;
   // row-major B: group c carries K rows [HK c, HK c + HK) of B, BN elements each; a copy moves KRC whole K rows, the
   // lane at LDS position (row, slot) fetching the piece that belongs there (see ring16_row_swizzle)
   constexpr int KRC = 1024 / (BN * ES), LPR = 64 / KRC;
-  const int N = g.N;
-  uint32_t voff_b[B_KC ? 1 : B_PW];
-  const char* b_ubase;
-  size_t b_copy_step = 0, b_group_step = 0;
-  if constexpr (B_KC) {
-    b_ubase = b_base_of(n0);
-  } else {
-    static_assert(B_KC || (KRC * BN * ES == 1024 && NW * B_PW * KRC == HK), "whole K rows per copy, a K step per group");
+  static_assert(B_KC || (KRC * BN * ES == 1024 && NW * B_PW * KRC == HK), "whole K rows per copy, a K step per group");
+  uint32_t voff_a[2][A_PW], voff_b[B_KC ? 2 : 1][B_PW];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+#pragma unroll
+    for (int t = 0; t < A_PW; t++) {
+      // RAGGED: rows past the end are fetched from the last row (an output depends on its own row of A and column
+      // of B only, and those past the end are not stored)
+      int r = 16 * (wave * A_PW + t) + 8 * par + ci;
+      if constexpr (RAGGED) r = min(m0 + r, g.M - 1) - m0;
+      voff_a[par][t] = (uint32_t)((size_t)r * K * ES + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+    }
+    if constexpr (B_KC) {
+#pragma unroll
+      for (int t = 0; t < B_PW; t++) {
+        int r = 16 * (wave * B_PW + t) + 8 * par + ci;
+        if constexpr (RAGGED) r = min(n0 + r, N - 1) - n0;
+        voff_b[par][t] = (uint32_t)((size_t)r * K * ES + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
+      }
+    }
+  }
+  size_t b_group_step = 0;
+  if constexpr (!B_KC) {
     const int last_piece = (N - n0) / EPV - 1;   // RAGGED: N is a multiple of EPV on this path, n0 < N
 #pragma unroll
     for (int t = 0; t < B_PW; t++) {
       const int kr = (wave * B_PW + t) * KRC + lane / LPR;   // K row within the group
       int piece = (lane % LPR) ^ ring16_row_swizzle<ES>(kr);
       if constexpr (RAGGED) piece = min(piece, last_piece);  // columns past the end: the last piece (not stored)
-      voff_b[t] = (uint32_t)(((size_t)(lane / LPR) * N + (size_t)(piece * EPV)) * ES);
+      voff_b[0][t] = (uint32_t)(((size_t)kr * N + (size_t)(piece * EPV)) * ES) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
     }
-    b_ubase = b_base_of(n0);
-    b_copy_step = (size_t)KRC * N * ES;
     b_group_step = (size_t)HK * N * ES;
   }
-  // RAGGED: rows past the end are fetched from the last row (an output depends on its own row of A and column of B
-  // only, and those past the end are not stored); the per-copy offsets are then relative to the tile's first row
-  uint32_t voff_ar[2][RAGGED ? A_PW : 1], voff_br[2][RAGGED && B_KC ? B_PW : 1];
-  const char* a_tile = reinterpret_cast<const char*>(g.A) + (size_t)m0 * K * ES + k_byte0;
-  const char* b_tile = reinterpret_cast<const char*>(g.B) + (size_t)n0 * K * ES + k_byte0;
-  if constexpr (RAGGED) {
-#pragma unroll
-    for (int par = 0; par < 2; par++) {
-#pragma unroll
-      for (int t = 0; t < A_PW; t++) {
-        const int rc = min(m0 + 16 * (wave * A_PW + t) + 8 * par + ci, g.M - 1) - m0;
-        voff_ar[par][t] = (uint32_t)((size_t)rc * K * ES + (size_t)((cs ^ ci ^ par) * 16));
-      }
-      if constexpr (B_KC) {
-#pragma unroll
-        for (int t = 0; t < B_PW; t++) {
-          const int rc = min(n0 + 16 * (wave * B_PW + t) + 8 * par + ci, g.N - 1) - n0;
-          voff_br[par][t] = (uint32_t)((size_t)rc * K * ES + (size_t)((cs ^ ci ^ par) * 16));
-        }
-      }
-    }
-  }
-  auto copy_a_begin = [&](int st) { asm_set_m0(lds_base + st * STAGE_BYTES + (wave * A_PW) * 1024 + (A_PW / 2) * 1024); };
-  auto copy_b_begin = [&](int st) {
-    asm_set_m0(lds_base + st * STAGE_BYTES + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024);
+  // scalar bases of a tile: its first row of A (first column of a K-contiguous B) at the first K byte of this run; a
+  // row-major B's first K row of the run at the tile's first column
+  auto a_base_of = [&](int m_first) -> const char* {
+    return reinterpret_cast<const char*>(g.A) + (size_t)m_first * K * ES + k_byte0 - COPY_BIAS;
   };
-  auto copy_a = [&](auto t_c, auto p_c, int c, uint64_t mask) {
+  auto b_base_of = [&](int n_first) -> const char* {
+    if constexpr (B_KC) return reinterpret_cast<const char*>(g.B) + (size_t)n_first * K * ES + k_byte0 - COPY_BIAS;
+    else return reinterpret_cast<const char*>(g.B) + ((size_t)(2 * slab0) * HK * N + n_first) * ES - COPY_BIAS;
+  };
+  // where copy group C of a tile starts, from the tile's bases
+  auto a_group = [&](const char* a_tile, int c) -> const char* { return a_tile + (size_t)(c >> 1) * LINE; };
+  auto b_group = [&](const char* b_tile, int c) -> const char* {
+    if constexpr (B_KC) return b_tile + (size_t)(c >> 1) * LINE;
+    else return b_tile + (size_t)c * b_group_step;
+  };
+  const uint32_t m0_a = lds_base + (wave * A_PW) * 1024 + (A_PW / 2) * 1024;
+  const uint32_t m0_b = lds_base + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024;
+  auto copy_a_begin = [&](int st) { asm_set_m0(m0_a + st * STAGE_BYTES); };
+  auto copy_b_begin = [&](int st) { asm_set_m0(m0_b + st * STAGE_BYTES); };
+  auto copy_a = [&](auto t_c, auto p_c, const char* src, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - A_PW / 2) * 1024;
-    if constexpr (RAGGED) asm_copy16_masked<OFF>(voff_ar[P][Tn], a_tile + (size_t)(c >> 1) * LINE - OFF, mask);
-    else asm_copy16_masked<OFF>(voff[P], a_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
+    asm_copy16_masked<OFF>(voff_a[P][Tn], src, mask);
   };
-  auto copy_b = [&](auto t_c, auto p_c, int c, uint64_t mask) {
+  auto copy_b = [&](auto t_c, auto p_c, const char* src, uint64_t mask) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - B_PW / 2) * 1024;
-    if constexpr (!B_KC) asm_copy16_masked<OFF>(voff_b[Tn], b_ubase + Tn * b_copy_step + (size_t)(2 * slab0 + c) * b_group_step - OFF, mask);
-    else if constexpr (RAGGED) asm_copy16_masked<OFF>(voff_br[P][Tn], b_tile + (size_t)(c >> 1) * LINE - OFF, mask);
-    else asm_copy16_masked<OFF>(voff[P], b_ubase + Tn * group_step + P * parity_step + (size_t)(c >> 1) * LINE - OFF, mask);
+    asm_copy16_masked<OFF>(voff_b[B_KC ? P : 0][Tn], src, mask);
   };
 
   // ---- fragment addressing: one LDS byte address per (slab position in the ring, K step) ----
@@ -343,10 +351,12 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 
   // One K step: NMMA MFMAs on register set SET, rows of blocks walked back and forth so that consecutive
   // instructions share an operand.  Between them the NRD fragment reads of (ring position RJ, K step SET ^ 1) into
-  // the other set, and the copies of group c (parity CP) into buffer cst: the A rows in the first half, the B rows
-  // in the second.
-  auto kstep = [&](auto set_c, auto rj_c, auto cp_c, int cst, int c, uint64_t cmask) {
-    constexpr int SET = decltype(set_c)::value;
+  // the other set, and the copies of a group of parity CP into buffer CST from a_src / b_src: the A rows in the first
+  // half, the B rows in the second.  The last two slabs of a run have nothing left to fetch: `mask` (the lanes of a
+  // copy, a scalar register pair) is zero there.  (One body for both cases: with a second instance of the step
+  // without copies the register allocator no longer kept the accumulators in place across the branches.)
+  auto kstep = [&](auto set_c, auto rj_c, auto cp_c, auto cst_c, uint64_t mask, const char* a_src, const char* b_src) {
+    constexpr int SET = decltype(set_c)::value, CST = decltype(cst_c)::value;
     constexpr int CPE = NMMA / NCP;                    // MFMAs per copy
     constexpr int RDE = (NMMA * 3 / 4) / NRD;          // MFMAs per read: the reads end with the third quarter of the step
     static_assert(CPE >= 2 && RDE >= 1 && NCP * CPE == NMMA, "a step's copies are spread evenly over its MFMAs");
@@ -365,11 +375,11 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       if constexpr (Q % RDE == RDE - 1 && Q / RDE < NRD)
         read_one(std::integral_constant<int, SET ^ 1>{}, std::integral_constant<int, Q / RDE>{}, rj_c);
       constexpr int Tc = Q / CPE;
-      if constexpr (Q == 0) copy_a_begin(cst);
-      if constexpr (Q == CPE * A_PW) copy_b_begin(cst);
+      if constexpr (Q == 0) copy_a_begin(CST);
+      if constexpr (Q == CPE * A_PW) copy_b_begin(CST);
       if constexpr (Q % CPE == CPE / 2) {
-        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, cp_c, c, cmask);
-        else copy_b(std::integral_constant<int, Tc - A_PW>{}, cp_c, c, cmask);
+        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, cp_c, a_src, mask);
+        else copy_b(std::integral_constant<int, Tc - A_PW>{}, cp_c, b_src, mask);
       }
     });
   };
@@ -419,9 +429,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       asm_mfma16_f8<TYPES>(acc[I][J], join8(join4(bh[0][J][0], bh[0][J][1]), join4(bh[1][J][0], bh[1][J][1])),
                            join8(af[0][I], af[1][I]));
   };
-  // half H of the slab at ring position JR; the copies of group c (parity H) into buffer cst as in kstep
-  auto half_f8 = [&](auto h_c, auto jr_c, int cst, int c, uint64_t cmask) {
-    constexpr int H = decltype(h_c)::value, JR = decltype(jr_c)::value;
+  // half H of the slab at ring position JR; the copies of a group of parity H into buffer CST as in kstep
+  auto half_f8 = [&](auto h_c, auto jr_c, auto cst_c, uint64_t mask, const char* a_src, const char* b_src) {
+    constexpr int H = decltype(h_c)::value, JR = decltype(jr_c)::value, CST = decltype(cst_c)::value;
     using NEXT = std::integral_constant<int, (JR + 1) % NST>;
     constexpr int CPE = HM / NCP;          // MFMAs per copy
     static_assert(CPE >= 2 && NCP * CPE == HM && FM == 8 && HM >= 16 && FN >= 3, "a half's copies and reads are spread over its MFMAs");
@@ -453,42 +463,51 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
           read_a_f8(std::integral_constant<int, (Q / 2) / 2>{}, std::integral_constant<int, (Q / 2) % 2>{}, NEXT{});
       }
       constexpr int Tc = Q / CPE;
-      if constexpr (Q == 0) copy_a_begin(cst);
-      if constexpr (Q == CPE * A_PW) copy_b_begin(cst);
+      if constexpr (Q == 0) copy_a_begin(CST);
+      if constexpr (Q == CPE * A_PW) copy_b_begin(CST);
       if constexpr (Q % CPE == CPE / 2) {
-        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, h_c, c, cmask);
-        else copy_b(std::integral_constant<int, Tc - A_PW>{}, h_c, c, cmask);
+        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, h_c, a_src, mask);
+        else copy_b(std::integral_constant<int, Tc - A_PW>{}, h_c, b_src, mask);
       }
     });
   };
 
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
-  // lane mask of a copy as a scalar register pair: all ones while the group exists, zero past the end
-  auto mask_if = [](bool on) -> uint64_t {
-    const uint32_t w = (uint32_t)__builtin_amdgcn_readfirstlane(on ? -1 : 0);
-    return ((uint64_t)w << 32) | w;
+  // lane mask of a copy as a scalar register pair: all ones while a < b, zero otherwise
+  auto mask_if_less = [](int a, int b) -> uint64_t {
+    uint64_t m;
+    asm volatile("s_cmp_lt_i32 %1, %2\n\ts_cselect_b64 %0, -1, 0" : "=s"(m) : "s"(a), "s"(b) : "scc");
+    return m;
   };
+  constexpr uint64_t ALL_LANES = ~0ull;
 
-  // ---- prologue: groups 0 .. 3 ----
-  auto issue_group = [&](auto c_c) {
+  // ---- prologue: groups 0 .. 3 (slabs 0 and 1; a run of one slab has groups 0 and 1 only) ----
+  const char* const a_tile = a_base_of(m0);
+  const char* const b_tile = b_base_of(n0);
+  auto issue_group = [&](auto c_c, const char* a_t, const char* b_t) {
     constexpr int C = decltype(c_c)::value;
-    const uint64_t m = mask_if(C < nc);
+    const char* const a_src = a_group(a_t, C);
+    const char* const b_src = b_group(b_t, C);
     copy_a_begin(C);
-    static_for<A_PW>([&](auto t) { copy_a(t, std::integral_constant<int, C & 1>{}, C, m); });
+    static_for<A_PW>([&](auto t) { copy_a(t, std::integral_constant<int, C & 1>{}, a_src, ALL_LANES); });
     copy_b_begin(C);
-    static_for<B_PW>([&](auto t) { copy_b(t, std::integral_constant<int, C & 1>{}, C, m); });
+    static_for<B_PW>([&](auto t) { copy_b(t, std::integral_constant<int, C & 1>{}, b_src, ALL_LANES); });
   };
-  if (PERSISTENT && prefetched) {   // groups 0 and 1 went out before the last tile's epilogue
-    issue_group(std::integral_constant<int, 2>{});
-    issue_group(std::integral_constant<int, 3>{});
-  } else {
-    static_for<4>([&](auto c_c) { issue_group(c_c); });
+  if (!(PERSISTENT && prefetched)) {   // (persistent: groups 0 and 1 went out before the last tile's epilogue)
+    issue_group(std::integral_constant<int, 0>{}, a_tile, b_tile);
+    issue_group(std::integral_constant<int, 1>{}, a_tile, b_tile);
   }
   // Slab 0 (groups 0 and 1) has landed; what was issued after it may still be on its way.  (Persistent: the last
   // epilogue's stores are counted between the two pairs of groups.  Loads return in order, so with no more than two
   // groups' worth of operations outstanding none of them can be a load of groups 0 and 1.)
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(2 * NCP) : "memory");
+  if (nc > 2) {
+    issue_group(std::integral_constant<int, 2>{}, a_tile, b_tile);
+    issue_group(std::integral_constant<int, 3>{}, a_tile, b_tile);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(2 * NCP) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  }
   if constexpr (F8) {   // lower rows of A and all but the last column of B of slab 0
     static_for<FM>([&](auto r_c) {
       constexpr int R = decltype(r_c)::value;
@@ -499,24 +518,32 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     static_for<NRD>([&](auto r) { read_one(I0{}, r, I0{}); });
   }
 
-  // ---- one slab; JR = j % 5 at compile time ----
+  // ---- one slab; JR = j % 5 at compile time.  Slab j fetches slab j + 2 (groups 2j + 4 and 2j + 5) from a_cp / b_cp ----
+  const char* a_cp = a_group(a_tile, 4);
+  const char* b_cp = b_group(b_tile, 4);
+  const int nslab = nc / 2;
   auto slab = [&](auto jr_c, int j) {
     constexpr int JR = decltype(jr_c)::value;
     using NEXT = std::integral_constant<int, (JR + 1) % NST>;
-    const int c4 = 2 * j + 4, c5 = 2 * j + 5;
-    if constexpr (F8) half_f8(I0{}, jr_c, (2 * JR + 4) % NST, c4, mask_if(c4 < nc));
-    else kstep(I0{}, jr_c, I0{}, (2 * JR + 4) % NST, c4, mask_if(c4 < nc));
-    if (c4 < nc) {  // the copies of group 2j+4 may stay in flight
+    using ST4 = std::integral_constant<int, (2 * JR + 4) % NST>;
+    using ST5 = std::integral_constant<int, (2 * JR + 5) % NST>;
+    const uint64_t mask = mask_if_less(j + 2, nslab);   // slab j + 2 exists
+    if constexpr (F8) half_f8(I0{}, jr_c, ST4{}, mask, a_cp, b_cp);
+    else kstep(I0{}, jr_c, I0{}, ST4{}, mask, a_cp, b_cp);
+    if (j + 2 < nslab) {  // the copies of group 2j+4 may stay in flight
       if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
-    if constexpr (F8) half_f8(I1{}, jr_c, (2 * JR + 5) % NST, c5, mask_if(c5 < nc));
-    else kstep(I1{}, NEXT{}, I1{}, (2 * JR + 5) % NST, c5, mask_if(c5 < nc));
+    if constexpr (!B_KC) b_cp += b_group_step;   // a row-major B: a group is a K step's rows
+    if constexpr (F8) half_f8(I1{}, jr_c, ST5{}, mask, a_cp, b_cp);
+    else kstep(I1{}, NEXT{}, I1{}, ST5{}, mask, a_cp, b_cp);
+    a_cp += LINE;
+    if constexpr (B_KC) b_cp += LINE;
+    else b_cp += b_group_step;
   };
 
-  const int nslab = nc / 2;
   for (int j = 0; j < nslab; j += NST) {
     slab(std::integral_constant<int, 0>{}, j);
     if (j + 1 < nslab) slab(std::integral_constant<int, 1>{}, j + 1);
@@ -543,9 +570,11 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     if (next_bid < tiles_m * tiles_n) {
       int tm2, tn2;
       tile_of_block(next_bid, tiles_m, tiles_n, tm2, tn2);
-      a_ubase = reinterpret_cast<const char*>(g.A) + (size_t)(tm2 * BM + 16 * wave * A_PW) * K * ES;
-      b_ubase = b_base_of(tn2 * BN);
-      static_for<2>([&](auto c_c) { issue_group(c_c); });   // into buffers 0 and 1, which the epilogue does not use
+      const char* const a_next = a_base_of(tm2 * BM);
+      const char* const b_next = b_base_of(tn2 * BN);
+      // into buffers 0 and 1, which the epilogue does not use
+      issue_group(std::integral_constant<int, 0>{}, a_next, b_next);
+      issue_group(std::integral_constant<int, 1>{}, a_next, b_next);
       prefetched = true;
     }
   }

@@ -124,7 +124,7 @@ typedef struct gz_plan_t {
    * that costs as much as a whole one; the last tail_cols columns then run in a second launch (tail_tile_*,
    * tail_grid describe it; 0: no such split; never together with tail_rows).                                  */
   int32_t tail_cols;
-  /* MFMA rung, stream-K (variants 10 and 11, and the launcher's choice where its estimate prefers it): the 256x256
+  /* MFMA rung, stream-K (variants 7 and 8, and the launcher's choice where its estimate prefers it): the 256x256
    * tiles past the last whole round of the compute units, streamk_tiles of them, have their K slabs dealt in equal
    * contiguous runs to streamk_blocks work-groups of the same launch (grid = whole tiles + streamk_blocks); every
    * run leaves partial sums in a workspace of workspace_bytes that the caller never sees, and a second launch
@@ -133,8 +133,12 @@ typedef struct gz_plan_t {
   int64_t workspace_bytes;
 } gz_plan_t;
 
-/* variant: 0 = launcher's choice; other values select a tile configuration of the rung
- * (see gz_plan / gz_variant_count).                                                  */
+/* variant: 0 = launcher's choice; other values select a tile configuration of the rung (1 .. gz_variant_count).
+ * MFMA rung: 1 256x256 on four waves, 2 on eight, 3 128x128, 4 256x128 (register-staged or compiler-scheduled
+ * direct-to-LDS kernels, any shape and layout); 5 / 6 the hand-scheduled 256x256 ring kernel on four / eight waves
+ * wherever the problem allows it (row-major A, whole K slabs, 16-byte aligned rows; otherwise the kernel of 1 / 2);
+ * 7 / 8 the same with the stream-K decomposition; 9 / 10 as 5 / 6 with one work-group per tile instead of one per
+ * compute unit.                                                                                                */
 int gz_gemm_s8s8s32(const int8_t* A, const int8_t* B, const int32_t* C, int32_t* D,
                     int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                     int32_t alpha, int32_t beta, int rung, int variant, gz_stream stream);
@@ -191,8 +195,11 @@ int gz_gemm(int types, const void* A, const void* B, const void* C, void* D,
  * not in the library's pool, which hipMalloc grows on demand, but in a buffer of GZ_STATIC_SCRATCH_BYTES (384
  * slots of 256 x 256 accumulators) that is part of the library's device image, so that every GPU the library runs
  * on holds its own copy until the process ends.  This entry point never allocates or frees.  A launch that would
- * need more (gz_plan_t.workspace_bytes says how much) returns GZ_ERR_UNSUPPORTED with both sizes in
- * gz_last_error(); the variants without stream-K (8, 9) never need any.  The buffer keeps the last call's contents;
+ * need more than that does not arise under the launcher's own choice (variant 0): there the launcher keeps to plans
+ * that fit (gz_plan_static_scratch reports them; they may differ from gz_plan's where gz_plan's workspace_bytes exceeds
+ * the buffer, and then the results agree with gz_gemm's within the type's tolerance instead of bit for bit).  An
+ * explicit stream-K variant (7, 8) that needs more returns GZ_ERR_UNSUPPORTED with both sizes in gz_last_error(); the
+ * variants without stream-K never need any.  The buffer keeps the last call's contents;
  * nothing in it has to start at zero, every slot is written before it is read.  All calls on one GPU share it:
  * calls that overlap in time on one GPU (two streams, two host threads) race on it and must be serialised by the
  * caller.                                                                                                       */
@@ -209,6 +216,11 @@ int gz_gemm_static_scratch(int types, const void* A, const void* B, const void* 
  * to get the geometry they will choose there.                                        */
 int gz_plan(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
             int rung, int variant, int num_cus, int lds_per_cu, gz_plan_t* plan);
+
+/* The same for gz_gemm_static_scratch: the launcher's choice (variant 0) keeps to plans whose workspace_bytes fit
+ * GZ_STATIC_SCRATCH_BYTES.  No counterpart in the reference.                                                    */
+int gz_plan_static_scratch(int types, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+                           int rung, int variant, int num_cus, int lds_per_cu, gz_plan_t* plan);
 
 /* The two device properties the functor constructors plan with (what nvidia/utils/benchmark.cuh:20-24 reads
  * into cudaDeviceProp for every functor): compute units and LDS bytes per compute unit of the device that is

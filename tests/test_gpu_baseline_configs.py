@@ -205,7 +205,7 @@ def test_mostly_empty_last_round_runs_as_two_launches(G, types, shape, lb):
         ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=rows)
         assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, shape, lb, rows)
     # the whole result against the single launch of the same tile (on-device compare would need both; host is enough)
-    one = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, 6)
+    one = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, 5)
     assert np.array_equal(got, one)
     # beta = 0 with no C
     got0 = G.run_gemm(types, ha, hb, None, m, n, k, O.ROW, lb, 1, 0, -1)
@@ -214,14 +214,14 @@ def test_mostly_empty_last_round_runs_as_two_launches(G, types, shape, lb):
 
 
 @pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.F16F16F16, O.E4M3E4M3F16])
-@pytest.mark.parametrize("variant", [8, 9])
+@pytest.mark.parametrize("variant", [5, 6])
 @pytest.mark.parametrize("shape,lb", [((4352, 4096, 3), O.COL), ((8192, 4096, 1), O.ROW), ((4096, 6144, 6), O.COL)])
 def test_more_tiles_than_compute_units_on_the_ring_kernel(G, types, variant, shape, lb):
     """272, 512 and 384 whole 256x256 tiles: past one round of the compute units the ring kernel is persistent - a
     work-group walks several tiles and asks for the next tile's first slab before it stores the current one.  K is
     1, 3 or 6 slabs, so the prefetched groups are all, most or a few of a tile's copies.  First and last rows, and
-    rows of tiles that are a work-group's second or third, against the oracle; everything against the older
-    one-tile-per-work-group kernel (variant 6)."""
+    rows of tiles that are a work-group's second or third, against the oracle; everything against the same kernel
+    launched with one work-group per tile (variants 9 and 10)."""
     m, n, slabs = shape
     k = slabs * 128 // np.dtype(O.IN_DTYPE[types]).itemsize
     kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
@@ -232,7 +232,7 @@ def test_more_tiles_than_compute_units_on_the_ring_kernel(G, types, variant, sha
     for rows in ((0, 4), (1020, 1028), (m // 2 - 2, m // 2 + 2), (m - 4, m)):
         ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=rows)
         assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, variant, shape, lb, rows)
-    one = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, 6)
+    one = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, variant + 4)
     assert np.array_equal(got, one)
 
 
