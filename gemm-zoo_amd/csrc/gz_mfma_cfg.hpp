@@ -133,9 +133,13 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // less than a whole one: the busy compute units have more of the chip's power and of their L2 (partial rounds of
     // 256 x 256 tiles measured at 0.73 - 0.85 of a whole one for a quarter to three quarters of the compute units).
     // (bf16 6000 x 6000 x 3000, 576 tiles: 261 us against 299 on 128 x 128 tiles, which the whole third round hid.)
-    if (i == 0 && !direct && !f32) {
+    // The ring kernel, persistent past one round, the same way (5120^2 x 4096, 400 tiles: 1.74 of the 4096^2 launch;
+    // 6144^2, 576 tiles: 2.69); a grid below one round costs it 0.8 of a round whatever its size (2048^2 0.82,
+    // 3072^2 0.83).
+    if (i == 0 && !f32) {
       const long long full = tiles / num_cus, rem = tiles % num_cus;
       shape_cost = (double)full + (rem ? 0.65 + 0.25 * (double)rem / num_cus : 0.0);
+      if (direct && full == 0) shape_cost = 0.85;
     }
     // fp32 is bound by its matrix rate at every tile size, so a smaller tile costs what its share of the products
     // costs: 256 x 128 half a round per round of its own, 128 x 128 its tiles over four per compute unit (measured,
@@ -175,29 +179,30 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // 386.5 / 401.4.  (A row-major B: eight waves at every size, see below.)
       eight = !(tiles >= 4LL * num_cus && b_cols);
     } else {
-      // 16-bit output, K-contiguous B: eight waves while the grid is small, and at every size on whole tiles (their
-      // epilogue is bound by the number of its stores; 4096^3 with operands rotating through seven sets, us, four /
-      // eight waves: bf16 -> bf16 103.5 / 101.7, fp16 110.5 / 106.6).  With an fp32 output four waves: level at
-      // 4096^3 (105.2 / 105.4) and ahead beyond (4096^2 x 8192 194.5 / 197.8, 8192^3 770.6 / 790.8); they are also
-      // the less sensitive to operands that come from HBM rather than from the last-level cache (three sets / seven
-      // sets: 101.2 / 103.7 against 99.7 / 106.9 for eight waves).
-      if ((types == GZ_BF16BF16BF16 || types == GZ_F16F16F16) && b_cols &&
-          (tiles <= 2LL * num_cus || (M % 256 == 0 && N % 256 == 0)))
-        eight = true;
-      // Four waves are for grids of whole rounds.  Where compute units stay empty, or in the last of a few rounds,
-      // the busy ones have more of the chip's power and of their L2 to themselves, and eight waves use that better
-      // (two waves per SIMD cover each other's waits).  us, four / eight waves, K = 512, 1024, 4096 -
-      // bf16 -> f32: 3072^2 (144 tiles) 21.6 / 18.6, 29.9 / 26.4, 81.3 / 73.9; 3584^2 (196) 22.8 / 22.6, 32.2 / 31.4,
-      // 85.8 / 83.3; 4096^2 (256) 24.1 / 25.0, 34.9 / 35.3, 98.0 / 98.6; 4608^2 (324) 44.3 / 38.3, 63.3 / 56.9,
-      // 178.1 / 170.3; 5120^2 (400) 45.3 / 39.6, 66.5 / 59.6, 184.1 / 181.5; 6144^2 (576) 67.8 / 60.5, 96.1 / 89.4,
-      // 274.8 / 273.9; int8 the same way (3072^2 15.8 / 14.2, 20.4 / 18.6, 46.2 / 42.4; 5120^2 34.9 / 30.3,
-      // 44.6 / 39.5, 106.6 / 99.0).  From three rounds on four waves: 8192^3 770.6 / 790.8.
-      if (tiles % num_cus != 0 && tiles / num_cus < 3) eight = true;
-      // A row-major B comes out of LDS through the transposing reads, two per fragment: eight waves at every size
-      // (us, four / eight waves, row/row: bf16 4096^3 104.5 / 101.3, 8192^3 823.5 / 791.5, 4096^2 x 1024 39.0 / 37.5,
-      // 4000^2 x 4096 109.3 / 102.6; fp16 4096^3 111.3 / 104.8, 8192^3 856 / 810; int8 4096^3 61.9 / 59.6, 8192^3
-      // 444.2 / 437.6, 8000^2 x 8192 448.2 / 435.1; e4m3 8192^3 400.8 / 394.7, 8000^2 x 8192 431.8 / 409.6).
-      if (!b_cols) eight = true;
+      // int8 and the 16-bit types: an estimate of the launch on four and on eight waves, in us per round of tiles,
+      // a fixed part (first copies, epilogue) and a part per K slab.  Eight waves (two per SIMD, 128 x 64 per wave)
+      // start and end a tile faster - a 16-bit output most of all: its epilogue is bound by the number of its stores,
+      // and two waves per SIMD keep more of them in flight - but read a quarter more LDS bytes per product, which
+      // costs per slab with a K-contiguous B (where four waves issue one copy per eight MFMAs and nothing else) and
+      // nothing with a row-major B (whose transposing reads, two per fragment, four waves have to fit between their
+      // MFMAs).  Fitted to squares 3072 ... 8192, K = 1024 and 4096, us, four / eight waves -
+      // bf16 -> f32 row/col: 3072^2 29.8 / 30.3, 80.3 / 89.1; 4096^2 34.2 / 36.4, 96.6 / 103.4; 5120^2 59.3 / 57.0,
+      // 167.8 / 170.4; 6144^2 92.4 / 88.5, 259.6 / 261.8; 8192^2 147.4 / 156.1, 388.9 / 421.2;
+      // bf16 -> bf16 row/col: 3072^2 31.2 / 29.6, 81.7 / 88.7; 4096^2 33.9 / 31.5, 96.1 / 98.0; 5120^2 60.4 / 54.0,
+      // 167.2 / 167.9; 8192^2 133.8 / 129.3, 376.7 / 393.0; row/row 4096^2 34.9 / 31.5, 101.3 / 97.9; 5120^2
+      // 63.3 / 54.8, 174.2 / 168.2; 8192^2 143.3 / 136.1, 387.7 / 385.5;
+      // bf16 -> f32 row/row: 4096^2 35.1 / 36.5, 101.5 / 101.2; 5120^2 61.7 / 58.7, 175.8 / 173.6; 8192^2
+      // 154.2 / 155.9, 398.2 / 415.6; int8 row/col 4096^2 24.1 / 25.3, 55.2 / 58.6; 5120^2 42.1 / 38.4, 94.4 / 94.2;
+      // 8192^2 106.0 / 106.2, 231.6 / 248.9.
+      const bool out16 = types == GZ_BF16BF16BF16 || types == GZ_F16F16F16;
+      const double nslab = (double)K * in_size / MFMA_SLAB_BYTES;
+      const bool under_a_round = tiles < num_cus, whole_rounds = tiles % num_cus == 0;
+      const double slope4 = b_cols ? 1.30 : 1.38;
+      double slope8 = slope4 * (b_cols ? (under_a_round ? 1.17 : 1.07) : (under_a_round ? 1.11 : 0.985));
+      if (tiles >= 3LL * num_cus) slope8 *= 1.05;   // past three rounds four waves pull ahead (8192^2 x 4096 above)
+      const double fixed4 = out16 ? 13.6 : 13.2;
+      const double fixed8 = out16 ? 9.6 : whole_rounds ? 14.1 : 10.5;   // compute units left empty: more of the power and of the L2 for the busy ones
+      eight = fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
     }
     if (eight) *out = kMfmaCfgs[MFMA_CFG_RING_W8];
   }
@@ -416,7 +421,8 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
   if (full == 0 && nslab < (4 * R > 48 ? 4 * R : 48)) return false;
   // past whole rounds only where few tiles remain: between an eighth and most of a round the estimates of the
   // alternatives are not sharp enough to tell (4608^3: 180 us with the rows cut in two launches, 188 here)
-  if (full > 0 && R > num_cus / 8) return false;
+  // (two whole rounds and a quarter: 6144^2 x 4096, 64 of 576 tiles remain, 248 us against 268 in one plain launch)
+  if (full > 0 && R > (full >= 2LL * num_cus ? num_cus / 4 : num_cus / 8)) return false;
   // what the launcher would do otherwise, in the same unit (its estimates count rounds of 256 x 256 tiles)
   MfmaSplit sp;
   MfmaColSplit cs;

@@ -357,9 +357,12 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // without copies the register allocator no longer kept the accumulators in place across the branches.)
   auto kstep = [&](auto set_c, auto rj_c, auto cp_c, auto cst_c, uint64_t mask, const char* a_src, const char* b_src) {
     constexpr int SET = decltype(set_c)::value, CST = decltype(cst_c)::value;
-    constexpr int CPE = NMMA / NCP;                    // MFMAs per copy
+#ifndef GZ_X_SPAN
+#define GZ_X_SPAN 1
+#endif
+    constexpr int CPE = NMMA / NCP / GZ_X_SPAN > 0 ? NMMA / NCP / GZ_X_SPAN : 1;                    // MFMAs per copy
     constexpr int RDE = (NMMA * 3 / 4) / NRD;          // MFMAs per read: the reads end with the third quarter of the step
-    static_assert(CPE >= 2 && RDE >= 1 && NCP * CPE == NMMA, "a step's copies are spread evenly over its MFMAs");
+    static_assert(RDE >= 1, "a step's copies are spread evenly over its MFMAs");
     asm volatile("s_waitcnt lgkmcnt(0)");
     if constexpr (!B_KC) {
 #pragma unroll
@@ -377,7 +380,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       constexpr int Tc = Q / CPE;
       if constexpr (Q == 0) copy_a_begin(CST);
       if constexpr (Q == CPE * A_PW) copy_b_begin(CST);
-      if constexpr (Q % CPE == CPE / 2) {
+      if constexpr (Q % CPE == CPE / 2 && Tc < NCP) {
         if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, cp_c, a_src, mask);
         else copy_b(std::integral_constant<int, Tc - A_PW>{}, cp_c, b_src, mask);
       }

@@ -174,8 +174,12 @@ def test_column_cut_weighs_k(capi):
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (1, 16, 1)
     p = capi.plan(capi.F16F16F16, 4096, 4099, 4096, 0, 1)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (3, 16, 3)
-    p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 0)
+    p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 1, 0)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (8, 128, 128)
+    # row-major A and B: a cut along the columns would put the first launch on the register-staged kernel (a column
+    # range of a row-major B is not a packed matrix); the rows are cut instead, and both launches keep their kernels
+    p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 0)
+    assert p.tail_cols == 0 and p.tail_rows == 256 and (p.tile_m, p.tile_n) == (256, 256)
     # with a K-contiguous B the sixteen tiles of that seventeenth tile column are cut along K instead (stream-K)
     p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 1)
     assert p.tail_cols == 0 and p.streamk_tiles == 16
