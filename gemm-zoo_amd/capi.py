@@ -39,7 +39,7 @@ EXPORTS = [
     "gz_gemm_s8s8s32", "gz_gemm_bf16bf16f32", "gz_gemm_bf16bf16bf16", "gz_gemm_f16f16f16", "gz_gemm_f32f32f32",
     "gz_gemm_e4m3e4m3f16", "gz_gemm_e5m2e5m2f16", "gz_gemm_bf16bf16bf16_acc16", "gz_gemm_f16f16f16_acc16", "gz_gemm",
     "gz_plan", "gz_variant_count", "gz_rung_name", "gz_types_name", "gz_fill", "gz_compare", "gz_compare_rel",
-    "gz_last_error", "gz_version", "gz_device_props", "gz_gemm_static_scratch", "gz_plan_static_scratch",
+    "gz_last_error", "gz_version", "gz_device_props", "gz_gemm_static_scratch", "gz_plan_static_scratch", "gz_gemm_ld",
 ]
 
 
@@ -83,6 +83,7 @@ def _load():
         getattr(lib, name).argtypes = common + [f32, f32, i32, i32, vp]
     lib.gz_gemm.argtypes = [i32] + common + [f64, f64, i32, i32, vp]
     lib.gz_gemm_static_scratch.argtypes = [i32] + common + [f64, f64, i32, i32, vp]
+    lib.gz_gemm_ld.argtypes = [i32, vp, i64, vp, i64, vp, i64, vp, i64, i64, i64, i64, i32, i32, f64, f64, i32, i32, vp]
     lib.gz_plan.argtypes = [i32, i64, i64, i64, i32, i32, i32, i32, i32, i32, C.POINTER(Plan)]
     lib.gz_plan_static_scratch.argtypes = lib.gz_plan.argtypes
     lib.gz_variant_count.argtypes = [i32, i32]
@@ -136,6 +137,14 @@ def gemm(types: int, a, b, c, d, m: int, n: int, k: int, layout_a: int = ROW_MAJ
     if types == S8S8S32:
         alpha, beta = int(alpha), int(beta)
     check(fn(_ptr(a), _ptr(b), _ptr(c), _ptr(d), m, n, k, layout_a, layout_b, alpha, beta, rung, variant, stream))
+
+
+def gemm_ld(types: int, a, lda: int, b, ldb: int, c, ldc: int, d, ldd: int, m: int, n: int, k: int,
+            layout_a: int = ROW_MAJOR, layout_b: int = ROW_MAJOR, alpha=1, beta=0, rung: int = RUNG_AUTO, variant: int = 0,
+            stream: int = 0) -> None:
+    """gz_gemm_ld: matrices with leading dimensions in elements, 0 = packed (raises GzError on a non-zero status)."""
+    check(lib.gz_gemm_ld(types, _ptr(a), lda, _ptr(b), ldb, _ptr(c), ldc, _ptr(d), ldd, m, n, k, layout_a, layout_b,
+                         float(alpha), float(beta), rung, variant, stream))
 
 
 STATIC_SCRATCH_BYTES = 96 << 20

@@ -140,11 +140,12 @@ static int check_problem(int types, int64_t M, int64_t N, int64_t K, int layoutA
     set_error("unknown rung %d", rung);
     return GZ_ERR_BAD_ARG;
   }
-  // kernels index with 32-bit element counts per matrix
+  // extents and leading dimensions are 32-bit in the kernels; every index they form from them is 64-bit, so a matrix
+  // may hold 2^31 elements and more
   const int64_t lim = (int64_t)1 << 31;
-  if (M >= lim || N >= lim || K >= lim || M * K >= lim || K * N >= lim || M * N >= lim) {
-    set_error("matrix with 2^31 or more elements is not supported (M=%lld N=%lld K=%lld)", (long long)M,
-              (long long)N, (long long)K);
+  if (M >= lim || N >= lim || K >= lim) {
+    set_error("an extent of 2^31 or more is not supported (M=%lld N=%lld K=%lld)", (long long)M, (long long)N,
+              (long long)K);
     return GZ_ERR_UNSUPPORTED;
   }
   return GZ_OK;
@@ -156,13 +157,35 @@ static int resolve_rung(int types, int64_t M, int64_t N, int64_t K, int layoutA,
   return GZ_RUNG_MFMA;
 }
 
+// Leading dimensions: 0 stands for the packed value; otherwise at least the line's extent and below 2^31.
+static int resolve_ld(const char* name, int64_t given, int64_t extent, int64_t* out) {
+  if (given == 0) given = extent > 0 ? extent : 1;
+  if (given < extent || given < 1) {
+    set_error("%s = %lld is smaller than the %lld elements of a line", name, (long long)given, (long long)extent);
+    return GZ_ERR_BAD_ARG;
+  }
+  if (given >= ((int64_t)1 << 31)) {
+    set_error("%s = %lld: a leading dimension of 2^31 or more is not supported", name, (long long)given);
+    return GZ_ERR_UNSUPPORTED;
+  }
+  *out = given;
+  return GZ_OK;
+}
+
+struct LeadingDims { int64_t a, b, c, d; };   // 0: packed
+
 template <int TYPES>
 static int run(const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K, int layoutA,
                int layoutB, typename Traits<TYPES>::scalar_t alpha, typename Traits<TYPES>::scalar_t beta, int rung,
-               int variant, gz_stream stream) {
+               int variant, gz_stream stream, LeadingDims ld = LeadingDims{0, 0, 0, 0}) {
   using T = Traits<TYPES>;
   int st = check_problem(TYPES, M, N, K, layoutA, layoutB, rung);
   if (st != GZ_OK) return st;
+  int64_t lda = 0, ldb = 0, ldc = 0, ldd = 0;
+  if ((st = resolve_ld("lda", ld.a, layoutA == GZ_ROW_MAJOR ? K : M, &lda)) != GZ_OK) return st;
+  if ((st = resolve_ld("ldb", ld.b, layoutB == GZ_ROW_MAJOR ? N : K, &ldb)) != GZ_OK) return st;
+  if ((st = resolve_ld("ldc", ld.c, N, &ldc)) != GZ_OK) return st;
+  if ((st = resolve_ld("ldd", ld.d, N, &ldd)) != GZ_OK) return st;
   if (M == 0 || N == 0) return GZ_OK;  // nothing to write
   if (!A && K > 0 && M > 0) { set_error("A is NULL"); return GZ_ERR_BAD_ARG; }
   if (!B && K > 0 && N > 0) { set_error("B is NULL"); return GZ_ERR_BAD_ARG; }
@@ -179,13 +202,13 @@ static int run(const void* A, const void* B, const void* C, void* D, int64_t M, 
   g.layoutA = layoutA; g.layoutB = layoutB;
   g.alpha = alpha; g.beta = beta;
   g.store_hint = 0;
-  g.ldb = g.ldd = (int)N;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   int resolved = resolve_rung(TYPES, M, N, K, layoutA, layoutB, rung);
-  // the streaming kernel needs 16-byte aligned operands; AUTO falls back to the tiled kernel otherwise
+  // the streaming kernel needs 16-byte aligned operands and lines; AUTO falls back to the tiled kernel otherwise
   if (rung == GZ_RUNG_AUTO && resolved == GZ_RUNG_SKINNY &&
-      ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15u))
+      (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15u) || !skinny_lines_ok(lda, ldb)))
     resolved = GZ_RUNG_MFMA;
   switch (resolved) {
     case GZ_RUNG_NAIVE: return launch_naive<TYPES>(g, variant, s);
@@ -264,8 +287,12 @@ int gz_gemm_f16f16f16_acc16(const uint16_t* A, const uint16_t* B, const uint16_t
                                  round_out<GZ_F16F16F16_ACC16>(beta), rung, variant, stream);
 }
 
-int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K,
-            int layoutA, int layoutB, double alpha, double beta, int rung, int variant, gz_stream stream) {
+// the typed launch behind gz_gemm and gz_gemm_ld (alpha and beta as doubles, rounded to the output type here as the
+// typed entry points do)
+static int gemm_any(int types, const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K,
+                    int layoutA, int layoutB, double alpha, double beta, int rung, int variant, gz_stream stream,
+                    LeadingDims ld) {
+  const float af = (float)alpha, bf = (float)beta;
   switch (types) {
     case GZ_S8S8S32:
       if (alpha != std::floor(alpha) || beta != std::floor(beta) || std::fabs(alpha) > 2147483647.0 ||
@@ -273,36 +300,40 @@ int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int
         set_error("s8s8s32 needs integral alpha/beta that fit int32");
         return GZ_ERR_BAD_ARG;
       }
-      return gz_gemm_s8s8s32((const int8_t*)A, (const int8_t*)B, (const int32_t*)C, (int32_t*)D, M, N, K, layoutA,
-                             layoutB, (int32_t)alpha, (int32_t)beta, rung, variant, stream);
-    case GZ_BF16BF16F32:
-      return gz_gemm_bf16bf16f32((const uint16_t*)A, (const uint16_t*)B, (const float*)C, (float*)D, M, N, K, layoutA,
-                                 layoutB, (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_BF16BF16BF16:
-      return gz_gemm_bf16bf16bf16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
-                                  layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_F16F16F16:
-      return gz_gemm_f16f16f16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
-                               layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_F32F32F32:
-      return gz_gemm_f32f32f32((const float*)A, (const float*)B, (const float*)C, (float*)D, M, N, K, layoutA, layoutB,
-                               (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_E4M3E4M3F16:
-      return gz_gemm_e4m3e4m3f16((const uint8_t*)A, (const uint8_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
-                                 layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_E5M2E5M2F16:
-      return gz_gemm_e5m2e5m2f16((const uint8_t*)A, (const uint8_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
-                                 layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_BF16BF16BF16_ACC16:
-      return gz_gemm_bf16bf16bf16_acc16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N,
-                                        K, layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
-    case GZ_F16F16F16_ACC16:
-      return gz_gemm_f16f16f16_acc16((const uint16_t*)A, (const uint16_t*)B, (const uint16_t*)C, (uint16_t*)D, M, N, K,
-                                     layoutA, layoutB, (float)alpha, (float)beta, rung, variant, stream);
+      return run<GZ_S8S8S32>(A, B, C, D, M, N, K, layoutA, layoutB, (int32_t)alpha, (int32_t)beta, rung, variant, stream, ld);
+    case GZ_BF16BF16F32: return run<GZ_BF16BF16F32>(A, B, C, D, M, N, K, layoutA, layoutB, af, bf, rung, variant, stream, ld);
+    case GZ_F32F32F32: return run<GZ_F32F32F32>(A, B, C, D, M, N, K, layoutA, layoutB, af, bf, rung, variant, stream, ld);
+#define GZ_ROUNDED(TY) \
+    case TY: return run<TY>(A, B, C, D, M, N, K, layoutA, layoutB, round_out<TY>(af), round_out<TY>(bf), rung, variant, stream, ld);
+    GZ_ROUNDED(GZ_BF16BF16BF16)
+    GZ_ROUNDED(GZ_F16F16F16)
+    GZ_ROUNDED(GZ_E4M3E4M3F16)
+    GZ_ROUNDED(GZ_E5M2E5M2F16)
+    GZ_ROUNDED(GZ_BF16BF16BF16_ACC16)
+    GZ_ROUNDED(GZ_F16F16F16_ACC16)
+#undef GZ_ROUNDED
     default: break;
   }
   set_error("unknown type bundle %d", types);
   return GZ_ERR_BAD_ARG;
+}
+
+int gz_gemm(int types, const void* A, const void* B, const void* C, void* D, int64_t M, int64_t N, int64_t K,
+            int layoutA, int layoutB, double alpha, double beta, int rung, int variant, gz_stream stream) {
+  return gemm_any(types, A, B, C, D, M, N, K, layoutA, layoutB, alpha, beta, rung, variant, stream,
+                  LeadingDims{0, 0, 0, 0});
+}
+
+int gz_gemm_ld(int types, const void* A, int64_t lda, const void* B, int64_t ldb, const void* C, int64_t ldc, void* D,
+               int64_t ldd, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB, double alpha, double beta,
+               int rung, int variant, gz_stream stream) {
+  if (lda < 0 || ldb < 0 || ldc < 0 || ldd < 0) {
+    set_error("negative leading dimension lda=%lld ldb=%lld ldc=%lld ldd=%lld", (long long)lda, (long long)ldb,
+              (long long)ldc, (long long)ldd);
+    return GZ_ERR_BAD_ARG;
+  }
+  return gemm_any(types, A, B, C, D, M, N, K, layoutA, layoutB, alpha, beta, rung, variant, stream,
+                  LeadingDims{lda, ldb, ldc, ldd});
 }
 
 int gz_device_props(int32_t* num_cus, int32_t* lds_per_cu) {

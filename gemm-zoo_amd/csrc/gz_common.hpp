@@ -93,10 +93,13 @@ template <int TYPES> struct GemmArgs {
   int layoutA, layoutB;
   typename T::scalar_t alpha, beta;
   int store_hint;   // MFMA rung, set by the launcher: bit 0 = the stores of D carry the non-temporal hint, bit 1 = the loads of C
-  // Row pitch in elements of a row-major B (ldb) and of C and D (ldd).  Both are N for every caller of the library;
-  // the MFMA launcher sets them apart from N when it runs a range of columns as a launch of its own, and only the
-  // kernels it then picks (register-staged tile kernel, 256x256 hand-scheduled kernel with K-contiguous B) read them.
-  int ldb, ldd;
+  // Leading dimensions in elements (nvidia/kernels/generic_gemm.cuh:6-8 takes the same four): the distance between
+  // consecutive lines of an operand - rows of a row-major A (at least K) or columns of a column-major one (at least
+  // M), K rows of a row-major B (at least N) or columns of a column-major one (at least K), rows of C and of D (at
+  // least N).  The packed entry points set them to those minima; the MFMA launcher also uses them to run a range of
+  // rows or columns of a problem as a launch of its own.  Every index is formed in 64 bits: a matrix may hold 2^31
+  // elements and more, its extents and leading dimensions stay below 2^31.
+  int64_t lda, ldb, ldc, ldd;
 };
 
 // ---------------------------------------------------------------------------

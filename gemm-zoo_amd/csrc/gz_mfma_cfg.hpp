@@ -138,7 +138,11 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // 3072^2 0.83).
     if (i == 0 && !f32) {
       const long long full = tiles / num_cus, rem = tiles % num_cus;
-      shape_cost = (double)full + (rem ? 0.65 + 0.25 * (double)rem / num_cus : 0.0);
+      const double frac = (double)rem / num_cus;
+      shape_cost = (double)full + (rem ? 0.65 + 0.25 * frac : 0.0);
+      // (the ring kernel: 0.72 of a round up to half a round of tiles, rising to a whole one - 4352 x 4096, 16 tiles
+      // left, 0.76; 6144^2, 64, 0.69; 5120^2, 144, 0.74; 5632^2, 228, 0.99)
+      if (direct && rem) shape_cost = (double)full + 0.72 + (frac > 0.5 ? 0.56 * (frac - 0.5) : 0.0);
       if (direct && full == 0) shape_cost = 0.85;
     }
     // fp32 is bound by its matrix rate at every tile size, so a smaller tile costs what its share of the products
@@ -441,12 +445,23 @@ inline long long mfma_persistent_grid(long long tiles, int num_cus) {
   return tiles > num_cus ? num_cus : tiles;
 }
 
-// Shape class of a launch: the direct-to-LDS kernels also need 16-byte aligned operands.
-inline int mfma_launch_class(const MfmaCfg& c, int in_size, int M, int N, int K, int layoutA, int layoutB, const void* A,
-                             const void* B, const void* C, const void* D) {
+// Shape class of a launch.  Beyond the extents, the direct-to-LDS kernels and the unpredicated register-staged one
+// need 16-byte aligned operands and lines (leading dimensions that are whole 16-byte pieces) and address a tile's
+// lines with 32-bit byte offsets from its first; the whole-tile epilogue stores 16 bytes per lane, so the rows of C and
+// D must be whole 16-byte pieces as well, or the launch takes the epilogue of the ragged kernels.
+inline int mfma_launch_class(const MfmaCfg& c, int in_size, int out_size, int M, int N, int K, int layoutA, int layoutB,
+                             const void* A, const void* B, const void* C, const void* D, long long lda, long long ldb,
+                             long long ldc, long long ldd) {
   const uintptr_t bits = (uintptr_t)A | (uintptr_t)B | (uintptr_t)C | (uintptr_t)D;
   if (bits & 15u) return MFMA_SHAPE_GENERAL;
-  return mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
+  if ((lda * in_size) % 16 || (ldb * in_size) % 16) return MFMA_SHAPE_GENERAL;
+  if (lda * in_size * 256 >= (1LL << 32) || ldb * in_size * 256 >= (1LL << 32)) return MFMA_SHAPE_GENERAL;
+  int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
+  if (cls == MFMA_SHAPE_WHOLE && ((ldd * out_size) % 16 || (C && (ldc * out_size) % 16))) {
+    const int epv = 16 / in_size;
+    cls = (layoutA == GZ_ROW_MAJOR && (layoutB == GZ_COL_MAJOR || N % epv == 0)) ? MFMA_SHAPE_RAGGED_MN : MFMA_SHAPE_GENERAL;
+  }
+  return cls;
 }
 
 }  // namespace gz

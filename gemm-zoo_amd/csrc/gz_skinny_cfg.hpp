@@ -48,6 +48,12 @@ inline bool skinny_supported(int types, int M, int N, int K, int layoutA, int la
   return K % SKINNY_K_STEP == 0;
 }
 
+// The streaming kernels copy 16-byte pieces of the rows of A and the columns of B and address them with 32-bit byte
+// offsets from the first row (column of the work-group): leading dimensions of whole pieces, below 2^32 / (2 * 128).
+inline bool skinny_lines_ok(long long lda, long long ldb) {
+  return lda % 8 == 0 && ldb % 8 == 0 && lda * 2 * SKINNY_MAX_M < (1LL << 32) && ldb * 2 * SKINNY_MAX_M < (1LL << 32);
+}
+
 // What the launcher's own choice sends here: always the register-resident cases; the LDS-shared tile kernel only
 // while the tiled MFMA rung could not give every compute unit a 128 x 128 tile of its own.
 inline bool skinny_preferred(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus) {

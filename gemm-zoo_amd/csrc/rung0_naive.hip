@@ -15,12 +15,11 @@ __global__ void __launch_bounds__(1024) naive_gemm_kernel(GemmArgs<TYPES> g) {
 
   RunningSum<TYPES> sum;
   for (int i = 0; i < g.K; i++) {
-    const auto a = widen_in<TYPES>(A_ROW ? g.A[(size_t)row * g.K + i] : g.A[(size_t)i * g.M + row]);
-    const auto b = widen_in<TYPES>(B_ROW ? g.B[(size_t)i * g.N + col] : g.B[(size_t)col * g.K + i]);
+    const auto a = widen_in<TYPES>(A_ROW ? g.A[(size_t)row * g.lda + i] : g.A[(size_t)i * g.lda + row]);
+    const auto b = widen_in<TYPES>(B_ROW ? g.B[(size_t)i * g.ldb + col] : g.B[(size_t)col * g.ldb + i]);
     sum.mac(a, b, i, g.K);
   }
-  const size_t o = (size_t)row * g.N + col;
-  g.D[o] = epilogue<TYPES>(sum.finish(g.K), g.alpha, g.beta, g.C + o);
+  g.D[(size_t)row * g.ldd + col] = epilogue<TYPES>(sum.finish(g.K), g.alpha, g.beta, g.C + (size_t)row * g.ldc + col);
 }
 
 template <int TYPES> int launch_naive(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {

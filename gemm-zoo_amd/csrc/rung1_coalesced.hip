@@ -29,8 +29,9 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
   RunningSum<TYPES> sum[TM];
 
   // 128-bit loads need every line start on a 16-byte boundary
-  const bool a_vec = A_KC && (K % EPV == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15u) == 0);
-  const bool b_vec = B_KC && (K % EPV == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15u) == 0);
+  const size_t lda = (size_t)g.lda, ldb = (size_t)g.ldb;
+  const bool a_vec = A_KC && (K % EPV == 0) && (lda % EPV == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15u) == 0);
+  const bool b_vec = B_KC && (K % EPV == 0) && (ldb % EPV == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15u) == 0);
 
   for (int k0 = 0; k0 < K; k0 += EPV) {
     in_t av[TM][EPV], bv[EPV];
@@ -40,7 +41,7 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
     for (int r = 0; r < TM; r++) {
       const int m = min(m0 + r, M - 1);
       if constexpr (A_KC) {
-        const in_t* p = g.A + (size_t)m * K + k0;
+        const in_t* p = g.A + (size_t)m * lda + k0;
         if (a_vec) {
           __builtin_memcpy(av[r], __builtin_assume_aligned(p, 16), 16);
         } else {
@@ -49,12 +50,12 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
         }
       } else {
 #pragma unroll
-        for (int e = 0; e < EPV; e++) av[r][e] = e < kn ? g.A[(size_t)(k0 + e) * M + m] : (in_t)0;
+        for (int e = 0; e < EPV; e++) av[r][e] = e < kn ? g.A[(size_t)(k0 + e) * lda + m] : (in_t)0;
       }
     }
     // ---- B ----
     if constexpr (B_KC) {
-      const in_t* p = g.B + (size_t)n_ld * K + k0;
+      const in_t* p = g.B + (size_t)n_ld * ldb + k0;
       if (b_vec) {
         __builtin_memcpy(bv, __builtin_assume_aligned(p, 16), 16);
       } else {
@@ -63,7 +64,7 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < EPV; e++) bv[e] = e < kn ? g.B[(size_t)(k0 + e) * N + n_ld] : (in_t)0;
+      for (int e = 0; e < EPV; e++) bv[e] = e < kn ? g.B[(size_t)(k0 + e) * ldb + n_ld] : (in_t)0;
     }
     // ---- multiply-accumulate in k order (zero-filled tail elements add exact zeros) ----
 #pragma unroll
@@ -82,8 +83,7 @@ __global__ void __launch_bounds__(256) coalesced_gemm_kernel(GemmArgs<TYPES> g) 
     for (int r = 0; r < TM; r++) {
       const int m = m0 + r;
       if (m < M) {
-        const size_t o = (size_t)m * N + n;
-        g.D[o] = epilogue<TYPES>(sum[r].finish((K + EPV - 1) / EPV * EPV), g.alpha, g.beta, g.C + o);
+        g.D[(size_t)m * g.ldd + n] = epilogue<TYPES>(sum[r].finish((K + EPV - 1) / EPV * EPV), g.alpha, g.beta, g.C + (size_t)m * g.ldc + n);
       }
     }
   }

@@ -28,27 +28,27 @@ template <int TYPES, bool KC> struct SlabLoader {
   using acc_t = typename Traits<TYPES>::acc_t;
   in_t r[8];
 
-  // base: matrix; lines_total: M or N; K; line0: first tile line; k0: first k of slab
-  __device__ inline void load(const in_t* __restrict__ base, int lines_total, int K, int line0, int k0, int tid,
+  // base: matrix; lines_total: M or N; K; ld: elements between its lines; line0: first tile line; k0: first k of slab
+  __device__ inline void load(const in_t* __restrict__ base, int lines_total, int K, size_t ld, int line0, int k0, int tid,
                               bool vec_ok) {
     if constexpr (KC) {
       const int line = line0 + (tid & 63), kk = k0 + (tid >> 6) * 8;
       if (line < lines_total && kk + 8 <= K && vec_ok) {
-        __builtin_memcpy(r, __builtin_assume_aligned(base + (size_t)line * K + kk, 8 * sizeof(in_t)), sizeof(r));
+        __builtin_memcpy(r, __builtin_assume_aligned(base + (size_t)line * ld + kk, 8 * sizeof(in_t)), sizeof(r));
       } else {
 #pragma unroll
         for (int e = 0; e < 8; e++)
-          r[e] = (line < lines_total && kk + e < K) ? base[(size_t)line * K + kk + e] : (in_t)0;
+          r[e] = (line < lines_total && kk + e < K) ? base[(size_t)line * ld + kk + e] : (in_t)0;
       }
     } else {
       const int kk = k0 + (tid >> 3), l0 = line0 + (tid & 7) * 8;
       if (kk < K && l0 + 8 <= lines_total && vec_ok) {
-        __builtin_memcpy(r, __builtin_assume_aligned(base + (size_t)kk * lines_total + l0, 8 * sizeof(in_t)),
+        __builtin_memcpy(r, __builtin_assume_aligned(base + (size_t)kk * ld + l0, 8 * sizeof(in_t)),
                          sizeof(r));
       } else {
 #pragma unroll
         for (int e = 0; e < 8; e++)
-          r[e] = (kk < K && l0 + e < lines_total) ? base[(size_t)kk * lines_total + l0 + e] : (in_t)0;
+          r[e] = (kk < K && l0 + e < lines_total) ? base[(size_t)kk * ld + l0 + e] : (in_t)0;
       }
     }
   }
@@ -84,8 +84,9 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
 
   // vector global loads need 8-element lines starting on their natural alignment
   constexpr uintptr_t VB = 8 * sizeof(in_t) - 1;
-  const bool a_vec = ((A_KC ? K : M) % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.A) & VB) == 0);
-  const bool b_vec = ((B_KC ? K : N) % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.B) & VB) == 0);
+  const size_t lda = (size_t)g.lda, ldb = (size_t)g.ldb;
+  const bool a_vec = ((A_KC ? K : M) % 8 == 0) && (lda % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.A) & VB) == 0);
+  const bool b_vec = ((B_KC ? K : N) % 8 == 0) && (ldb % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.B) & VB) == 0);
 
   SlabLoader<TYPES, A_KC> la;
   SlabLoader<TYPES, B_KC> lb;
@@ -110,8 +111,8 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
 
   if constexpr (STAGES == 1) {
     for (int t = 0; t < slabs; t++) {
-      la.load(g.A, M, K, m0, t * LT_BK, tid, a_vec);
-      lb.load(g.B, N, K, n0, t * LT_BK, tid, b_vec);
+      la.load(g.A, M, K, lda, m0, t * LT_BK, tid, a_vec);
+      lb.load(g.B, N, K, ldb, n0, t * LT_BK, tid, b_vec);
       la.store(lds, tid);
       lb.store(lds + SLAB, tid);
       __syncthreads();
@@ -120,8 +121,8 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
     }
   } else {
     if (slabs > 0) {
-      la.load(g.A, M, K, m0, 0, tid, a_vec);
-      lb.load(g.B, N, K, n0, 0, tid, b_vec);
+      la.load(g.A, M, K, lda, m0, 0, tid, a_vec);
+      lb.load(g.B, N, K, ldb, n0, 0, tid, b_vec);
       la.store(lds, tid);
       lb.store(lds + SLAB, tid);
     }
@@ -131,8 +132,8 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
       acc_t* nxt = lds + ((t + 1) & 1) * 2 * SLAB;
       const bool more = t + 1 < slabs;
       if (more) {  // global loads in flight while the FMAs below run
-        la.load(g.A, M, K, m0, (t + 1) * LT_BK, tid, a_vec);
-        lb.load(g.B, N, K, n0, (t + 1) * LT_BK, tid, b_vec);
+        la.load(g.A, M, K, lda, m0, (t + 1) * LT_BK, tid, a_vec);
+        lb.load(g.B, N, K, ldb, n0, (t + 1) * LT_BK, tid, b_vec);
       }
       compute(cur, cur + SLAB, K - t * LT_BK);
       if (more) {
@@ -151,8 +152,7 @@ __global__ void __launch_bounds__(LT_NT, 4) lds_gemm_kernel(GemmArgs<TYPES> g) {
     for (int j = 0; j < 4; j++) {
       const int n = n0 + tx * 4 + j;
       if (n < N) {
-        const size_t o = (size_t)m * N + n;
-        g.D[o] = epilogue<TYPES>(sum[i][j].finish(0), g.alpha, g.beta, g.C + o);
+        g.D[(size_t)m * g.ldd + n] = epilogue<TYPES>(sum[i][j].finish(0), g.alpha, g.beta, g.C + (size_t)m * g.ldc + n);
       }
     }
   }

@@ -106,7 +106,7 @@ __device__ inline typename AccVec<TYPES>::type mfma32(u32x4_t first, u32x4_t sec
 template <int TYPES, int FM, int FN, class Acc>
 __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc (&acc)[FM][FN], int row0, int col0, int lane) {
   using out_t = typename Traits<TYPES>::out_t;
-  const int LDD = g.ldd;
+  const size_t LDC = (size_t)g.ldc, LDD = (size_t)g.ldd;
   const bool use_c = g.beta != 0;
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
@@ -119,7 +119,7 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
         const size_t o = (size_t)m * LDD + n;
         const Acc& a = acc[I][J];
         out_t cv[4] = {0, 0, 0, 0}, dv[4];
-        if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+        if (use_c) __builtin_memcpy(cv, g.C + (size_t)m * LDC + n, sizeof(cv));
         dv[0] = epilogue<TYPES>(a[4 * Q + 0], g.alpha, g.beta, &cv[0]);
         dv[1] = epilogue<TYPES>(a[4 * Q + 1], g.alpha, g.beta, &cv[1]);
         dv[2] = epilogue<TYPES>(a[4 * Q + 2], g.alpha, g.beta, &cv[2]);
@@ -153,7 +153,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   // 17.7 with an fp32 output of 64 MiB).
   constexpr int W = (!RAGGED && sizeof(out_t) == 2) ? 8 : 4, WB = W * (int)sizeof(out_t);
   constexpr int LPR = COLS / W, RPI = 64 / LPR, NI = 32 / RPI;   // lanes per row, rows per instruction, instructions
-  const int M = g.M, N = g.N, LDD = g.ldd;   // LDD: elements between the rows of C and D (N unless the launch covers a column range)
+  const int M = g.M, N = g.N;
+  const size_t LDC = (size_t)g.ldc, LDD = (size_t)g.ldd;   // elements between the rows of C and of D
   const bool use_c = g.beta != 0;
   char* wr = BLK == 32 ? region + (lane & 31) * PITCH_E + (lane >> 5) * 16 : region + (lane & 15) * PITCH_E + (lane >> 4) * 16;
   const char* rd = region + (lane / LPR) * PITCH_E + (lane % LPR) * W * 4;
@@ -163,7 +164,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   // otherwise the block is written one element per lane with the lanes along a row, which is still whole cache
   // lines per instruction (fp16 4095 x 4097 x 63 took 65 us with four scattered 2-byte stores per lane).
   constexpr uintptr_t VEC_ALIGN = 4 * sizeof(out_t) - 1;
-  const bool vec = !RAGGED || ((N & 3) == 0 && (LDD & 3) == 0 && ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & VEC_ALIGN) == 0);
+  const bool vec = !RAGGED || ((N & 3) == 0 && (LDD & 3) == 0 && (!use_c || (LDC & 3) == 0) &&
+                               ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & VEC_ALIGN) == 0);
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
     // the block's values of C first: their latency passes while the accumulators go through LDS
@@ -176,14 +178,14 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       if (use_c && vec && (!RAGGED || (m < M && n < N))) {
         if (g.store_hint & 2) {   // non-temporal: see mfma_store_hint
           if constexpr (WB == 16) {
-            const u32x4_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.C + (size_t)m * LDD + n));
+            const u32x4_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.C + (size_t)m * LDC + n));
             __builtin_memcpy(cv[T], &w, 16);
           } else {
-            const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(g.C + (size_t)m * LDD + n));
+            const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(g.C + (size_t)m * LDC + n));
             __builtin_memcpy(cv[T], &w, 8);
           }
         } else {
-          __builtin_memcpy(cv[T], g.C + (size_t)m * LDD + n, sizeof(cv[T]));
+          __builtin_memcpy(cv[T], g.C + (size_t)m * LDC + n, sizeof(cv[T]));
         }
       }
     });
@@ -259,8 +261,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
           static_for<NC>([&](auto c_c) {
             constexpr int C = decltype(c_c)::value;
             const int nn = col0 + C * 64 + lane;
-            const size_t o = (size_t)m * LDD + nn;
-            if (m < M && nn < N) g.D[o] = epilogue<TYPES>(v[R][C], g.alpha, g.beta, g.C + o);
+            if (m < M && nn < N) g.D[(size_t)m * LDD + nn] = epilogue<TYPES>(v[R][C], g.alpha, g.beta, g.C + (size_t)m * LDC + nn);
           });
         });
       }
@@ -297,7 +298,7 @@ constexpr int KSTEPS = SLAB_BYTES / 32;   // MFMA steps per slab
 // matrix whose lines are `extent` long and `pitch` elements apart.  With EDGE the access is predicated and
 // zero-filled, and may be unaligned (gfx950 global loads tolerate that).
 template <typename in_t, bool EDGE>
-__device__ inline u32x4_t load16(const in_t* __restrict__ base, int line, int lines, int pos, int extent, int pitch) {
+__device__ inline u32x4_t load16(const in_t* __restrict__ base, int line, int lines, int pos, int extent, size_t pitch) {
   constexpr int EPV = 16 / (int)sizeof(in_t);
   if constexpr (!EDGE) {
     return *reinterpret_cast<const u32x4_t*>(base + (size_t)line * pitch + pos);
@@ -395,8 +396,8 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
   // bytes of one staged slab of this operand
   static constexpr int LDS_BYTES = (!KC && ES == 4) ? BK * NAT_PITCH : ROWS * PITCH;
 
-  // rows_total: M or N ; row0: first tile row ; k0: first k of the slab ; pitch: elements between the k lines of an
-  // operand whose lines run along M / N (rows_total unless the launch covers a range of columns of a wider matrix)
+  // rows_total: M or N ; row0: first tile row ; k0: first k of the slab ; pitch: the operand's leading dimension
+  // (elements between its lines: tile rows of a K-contiguous operand, k lines of one whose lines run along M / N)
   // The same for a slab whose k lines lie inside the matrix: k0 + BK <= K.  Every load is unconditional.  Lines of
   // the tile past the last row or column of the matrix are read from the last one instead: what is computed from
   // them is never stored, so it may be anything.  An operand whose lines run along M / N reads a 16-byte piece that
@@ -404,13 +405,13 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
   // slab must not hold the last k line of the matrix (k0 + BK <= K - 1).  The predicated loads of load() each end in a merge of
   // the loaded value with zero, and the compiler waits for a load at such a merge: eight loads per slab, one after
   // the other behind eight waits (fp16 4095 x 4096 x 1023 row/row: 57 us, of which the waits were a third).
-  __device__ inline void load_inside(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid, int pitch) {
+  __device__ inline void load_inside(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid, size_t pitch) {
     if constexpr (KC) {
 #pragma unroll
       for (int it = 0; it < VECS; it++) {
         const int id = it * NT + tid;
         const int row = min(row0 + (id >> 3), rows_total - 1), c = id & 7;
-        __builtin_memcpy(&r[it], base + (size_t)row * K + k0 + c * EPV, 16);
+        __builtin_memcpy(&r[it], base + (size_t)row * pitch + k0 + c * EPV, 16);
       }
     } else {
 #pragma unroll
@@ -423,13 +424,13 @@ template <typename in_t, int ROWS, int NT, bool KC, bool EDGE> struct Stager {
       }
     }
   }
-  __device__ inline void load(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid, int pitch) {
+  __device__ inline void load(const in_t* __restrict__ base, int rows_total, int K, int row0, int k0, int tid, size_t pitch) {
     if constexpr (KC) {
 #pragma unroll
       for (int it = 0; it < VECS; it++) {
         const int id = it * NT + tid;
         const int row = id >> 3, c = id & 7;
-        r[it] = load16<in_t, EDGE>(base, row0 + row, rows_total, k0 + c * EPV, K, K);
+        r[it] = load16<in_t, EDGE>(base, row0 + row, rows_total, k0 + c * EPV, K, pitch);
       }
     } else {
 #pragma unroll
@@ -613,7 +614,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr bool PEEL = EDGE;
   const bool ragged_lines = (!A_KC && m0 + BM > g.M) || (!B_KC && n0 + BN > g.N);
   // (lines shorter than a 16-byte piece: a piece could reach further than the next k line, so no such slabs)
-  const bool short_lines = (!A_KC && g.M < 16) || (!B_KC && g.ldb < 16);
+  const bool short_lines = (!A_KC && g.lda < 16) || (!B_KC && g.ldb < 16);
   const int full_slabs = ragged_lines ? (short_lines ? 0 : (g.K - 1) / BK) : g.K / BK;
   // how a slab is loaded: predicated, unconditionally (inside), or not at all (the last two iterations of the edge
   // kernels have no slab left to ask for; the registers keep what they hold and what is stored from them is never read)
@@ -623,11 +624,11 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   auto load_slab = [&](auto mode_c, int k0) __attribute__((always_inline)) {
     constexpr int MODE = decltype(mode_c)::value;
     if constexpr (MODE == 1) {
-      sa.load_inside(g.A, g.M, g.K, m0, k0, tid, g.M);
-      sb.load_inside(g.B, g.N, g.K, n0, k0, tid, g.ldb);
+      sa.load_inside(g.A, g.M, g.K, m0, k0, tid, (size_t)g.lda);
+      sb.load_inside(g.B, g.N, g.K, n0, k0, tid, (size_t)g.ldb);
     } else if constexpr (MODE == 0) {
-      sa.load(g.A, g.M, g.K, m0, k0, tid, g.M);
-      sb.load(g.B, g.N, g.K, n0, k0, tid, g.ldb);
+      sa.load(g.A, g.M, g.K, m0, k0, tid, (size_t)g.lda);
+      sb.load(g.B, g.N, g.K, n0, k0, tid, (size_t)g.ldb);
     }
   };
   auto load_slab_checked = [&](int slab) __attribute__((always_inline)) {
@@ -808,32 +809,32 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   const in_t* b_src[2];
   // row-major B: the slab is BK K rows of BN elements; a copy moves KRC whole rows, LPR lanes per row
   constexpr int TR_PITCH = BN * ES, KRC = 1024 / TR_PITCH, LPR = 64 / KRC, PPR = TR_PITCH / 16;
-  const int N = g.N;
+  const size_t LDA = (size_t)g.lda, LDB = (size_t)g.ldb;
 #pragma unroll
   for (int par = 0; par < 2; par++) {
     const int ca = lp ^ lr ^ (((wave * A_PW) & 1) ^ par);
     const int cb = lp ^ lr ^ (((wave * B_PW) & 1) ^ par);
-    a_src[par] = g.A + (size_t)(m0 + 8 * wave * A_PW + lr) * K + ca * EPV;
+    a_src[par] = g.A + (size_t)(m0 + 8 * wave * A_PW + lr) * LDA + ca * EPV;
     if constexpr (B_KC) {
-      b_src[par] = g.B + (size_t)(n0 + 8 * wave * B_PW + lr) * K + cb * EPV;
+      b_src[par] = g.B + (size_t)(n0 + 8 * wave * B_PW + lr) * LDB + cb * EPV;
     } else {
       static_assert(B_KC || (KRC >= 4 && KRC * TR_PITCH == 1024), "the swizzle of a row must not depend on the copy index");
       const int kr = lane / LPR;  // row within the copy; rows of a copy start at a multiple of KRC >= 4 (8 for int8)
-      b_src[par] = g.B + (size_t)(wave * B_PW * KRC + kr) * N + n0 + ((lane % LPR) ^ dtl_tr_swz<ES, PPR>(kr)) * EPV;
+      b_src[par] = g.B + (size_t)(wave * B_PW * KRC + kr) * LDB + n0 + ((lane % LPR) ^ dtl_tr_swz<ES, PPR>(kr)) * EPV;
     }
   }
   auto copy_slab = [&](char* stage, int k0) {
 #pragma unroll
     for (int t = 0; t < A_PW; t++)
-      __builtin_amdgcn_global_load_lds((gptr_t)(a_src[t & 1] + (size_t)(8 * t) * K + k0),
+      __builtin_amdgcn_global_load_lds((gptr_t)(a_src[t & 1] + (size_t)(8 * t) * LDA + k0),
                                        (lptr_t)(stage + (wave * A_PW + t) * 1024), 16, 0, 0);
 #pragma unroll
     for (int t = 0; t < B_PW; t++) {
       if constexpr (B_KC)
-        __builtin_amdgcn_global_load_lds((gptr_t)(b_src[t & 1] + (size_t)(8 * t) * K + k0),
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_src[t & 1] + (size_t)(8 * t) * LDB + k0),
                                          (lptr_t)(stage + A_BYTES + (wave * B_PW + t) * 1024), 16, 0, 0);
       else
-        __builtin_amdgcn_global_load_lds((gptr_t)(b_src[0] + (size_t)(k0 + KRC * t) * N),
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_src[0] + (size_t)(k0 + KRC * t) * LDB),
                                          (lptr_t)(stage + A_BYTES + (wave * B_PW + t) * 1024), 16, 0, 0);
     }
   };
@@ -1104,7 +1105,8 @@ __global__ void __launch_bounds__(STRIP_WAVES * 64) mfma_strip_kernel(GemmArgs<T
   __shared__ __attribute__((aligned(16))) in_t bs[R * K_CHUNK];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m0 = blockIdx.x * STRIP_ROWS_PER_WG + wave * STRIP_ROWS_PER_WAVE;
-  const int K = g.K, M = g.M, r = g.N, ldb = g.ldb;
+  const int K = g.K, M = g.M, r = g.N;
+  const size_t lda = (size_t)g.lda, ldb = (size_t)g.ldb;
   acc_t acc[STRIP_ROWS_PER_WAVE][R];
 #pragma unroll
   for (int i = 0; i < STRIP_ROWS_PER_WAVE; i++)
@@ -1164,13 +1166,13 @@ __global__ void __launch_bounds__(STRIP_WAVES * 64) mfma_strip_kernel(GemmArgs<T
         a[i][t] = u32x4_t{0, 0, 0, 0};
         if (kc0 + t * 64 * EPV >= k_vec_end) continue;
         if constexpr (A_KC) {
-          __builtin_memcpy(&a[i][t], g.A + (size_t)m * K + min(k, k_vec_end - EPV), 16);
+          __builtin_memcpy(&a[i][t], g.A + (size_t)m * lda + min(k, k_vec_end - EPV), 16);
         } else {
           u32x4_t v = {0, 0, 0, 0};
 #pragma unroll
           for (int e = 0; e < EPV; e++) {
             const int kk = min(k + e, K - 1);
-            v[e / EPW] |= elem_bits(g.A[(size_t)kk * M + m]) << (e % EPW * EBITS);
+            v[e / EPW] |= elem_bits(g.A[(size_t)kk * lda + m]) << (e % EPW * EBITS);
           }
           a[i][t] = v;
         }
@@ -1183,7 +1185,7 @@ __global__ void __launch_bounds__(STRIP_WAVES * 64) mfma_strip_kernel(GemmArgs<T
         tmp[t] = (in_t)0;
         if (t * STRIP_WAVES * 64 >= kn) continue;   // (the same for all lanes)
         const int kk = min(kc0 + (int)threadIdx.x + t * STRIP_WAVES * 64, K - 1);
-        tmp[t] = B_KC ? g.B[(size_t)j * K + kk] : g.B[(size_t)kk * ldb + j];
+        tmp[t] = B_KC ? g.B[(size_t)j * ldb + kk] : g.B[(size_t)kk * ldb + j];
       }
 #pragma unroll
       for (int t = 0; t < GI; t++) {
@@ -1230,11 +1232,11 @@ __global__ void __launch_bounds__(STRIP_WAVES * 64) mfma_strip_kernel(GemmArgs<T
       static_for<R>([&](auto j_c) {
         constexpr int j = decltype(j_c)::value;
         if (j < r) {
-          const in_t bv = B_KC ? g.B[(size_t)j * K + kk] : g.B[(size_t)kk * ldb + j];
+          const in_t bv = B_KC ? g.B[(size_t)j * ldb + kk] : g.B[(size_t)kk * ldb + j];
           const acc_t bw = mine ? widen_in<TYPES>(bv) : (acc_t)0;
 #pragma unroll
           for (int i = 0; i < STRIP_ROWS_PER_WAVE; i++) {
-            const in_t av = g.A[(size_t)min(m0 + i, M - 1) * K + kk];
+            const in_t av = g.A[(size_t)min(m0 + i, M - 1) * lda + kk];
             acc[i][j] = mac(mine ? widen_in<TYPES>(av) : (acc_t)0, bw, acc[i][j]);
           }
         }
@@ -1251,8 +1253,7 @@ __global__ void __launch_bounds__(STRIP_WAVES * 64) mfma_strip_kernel(GemmArgs<T
 #pragma unroll
       for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
       if (lane == 0 && j < r) {
-        const size_t o = (size_t)m * g.ldd + j;
-        g.D[o] = epilogue<TYPES>(v, g.alpha, g.beta, g.C + o);
+        g.D[(size_t)m * g.ldd + j] = epilogue<TYPES>(v, g.alpha, g.beta, g.C + (size_t)m * g.ldc + j);
       }
     }
   }
@@ -1279,11 +1280,8 @@ template <int TYPES> static int launch_strip(const GemmArgs<TYPES>& g, hipStream
 template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& chosen, hipStream_t s, bool adjust = false) {
   using in_t = typename Traits<TYPES>::in_t;
   MfmaCfg cfg = chosen;
-  int edge = mfma_launch_class(cfg, (int)sizeof(in_t), g.M, g.N, g.K, g.layoutA, g.layoutB, g.A, g.B, g.C, g.D);
-  // a column range of wider matrices: only the register-staged kernel reads the pitch of a row-major B, and the
-  // epilogue that reads the pitch of C and D unaligned is the one of the ragged kernels
-  if (g.layoutB == GZ_ROW_MAJOR && g.ldb != g.N) edge = MFMA_SHAPE_GENERAL;
-  else if (g.ldd != g.N && edge == MFMA_SHAPE_WHOLE) edge = MFMA_SHAPE_RAGGED_MN;
+  const int edge = mfma_launch_class(cfg, (int)sizeof(in_t), (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N, g.K,
+                                     g.layoutA, g.layoutB, g.A, g.B, g.C, g.D, g.lda, g.ldb, g.ldc, g.ldd);
   if (adjust) mfma_adjust_general(TYPES, edge, g.layoutA, &cfg);   // launcher's choice: the wave count follows the kernel
   switch (cfg.id) {
     case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
@@ -1336,15 +1334,16 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
   GemmArgs<TYPES> g = args;
   const int num_cus = device_compute_units();
   g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), num_cus);
-  if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && g.K > 0 && g.ldd == g.N) {
+  if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && g.K > 0) {
     StreamKPlan skp;
     const MfmaCfg* forced = variant == 0 ? nullptr : &kMfmaCfgs[variant - 1];
     // the launcher's own choice stays within the workspace this entry point may use (the entry point that
     // allocates nothing has a fixed one); an explicit stream-K variant is refused by workspace_acquire instead
     if (mfma_plan_streamk(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, num_cus, forced != nullptr, forced, &skp) &&
         (forced || (size_t)skp.slots * MFMA_STREAMK_SLOT_BYTES <= workspace_limit())) {
-      const int cls = mfma_launch_class(skp.cfg, (int)sizeof(typename Traits<TYPES>::in_t), g.M, g.N, g.K, g.layoutA,
-                                        g.layoutB, g.A, g.B, g.C, g.D);
+      const int cls = mfma_launch_class(skp.cfg, (int)sizeof(typename Traits<TYPES>::in_t),
+                                        (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N, g.K, g.layoutA, g.layoutB,
+                                        g.A, g.B, g.C, g.D, g.lda, g.ldb, g.ldc, g.ldd);
       if (cls != MFMA_SHAPE_GENERAL) {   // (unaligned operands: the plain launch below, on the register-staged kernel)
         g.store_hint = 0;   // one round at most ends in each launch: plain stores
         return skp.cfg.waves_n == 4 ? launch_streamk<TYPES, 4>(g, skp, cls == MFMA_SHAPE_RAGGED_MN, s)
@@ -1361,9 +1360,9 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       GemmArgs<TYPES> top = g, bottom = g;
       top.M = sp.rows_main;
       bottom.M = g.M - sp.rows_main;
-      bottom.A = g.A + (size_t)sp.rows_main * g.K;   // row-major A: a row range is a packed matrix
-      if (g.C) bottom.C = g.C + (size_t)sp.rows_main * g.N;
-      bottom.D = g.D + (size_t)sp.rows_main * g.N;
+      bottom.A = g.A + (size_t)sp.rows_main * (size_t)g.lda;   // row-major A: a row range is a matrix with the same pitch
+      if (g.C) bottom.C = g.C + (size_t)sp.rows_main * (size_t)g.ldc;
+      bottom.D = g.D + (size_t)sp.rows_main * (size_t)g.ldd;
       const int st = launch_one<TYPES>(top, sp.main, s, true);
       if (st != GZ_OK) return st;
       return launch_one<TYPES>(bottom, sp.tail, s, true);
@@ -1373,7 +1372,7 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
       GemmArgs<TYPES> left = g, right = g;
       left.N = cs.cols_main;
       right.N = g.N - cs.cols_main;
-      right.B = g.layoutB == GZ_ROW_MAJOR ? g.B + cs.cols_main : g.B + (size_t)cs.cols_main * g.K;
+      right.B = g.layoutB == GZ_ROW_MAJOR ? g.B + cs.cols_main : g.B + (size_t)cs.cols_main * (size_t)g.ldb;
       if (g.C) right.C = g.C + cs.cols_main;
       right.D = g.D + cs.cols_main;
       const int st = launch_one<TYPES>(left, cs.main, s, true);

@@ -24,11 +24,11 @@ typedef _Float16 a16_f16x4_t __attribute__((ext_vector_type(4)));
 // Eight consecutive k of one line (row of A / column of B) starting at k0, zero-filled outside the matrix.
 // KC: the line is contiguous in memory (row-major A, column-major B); `vec`: 16-byte loads are allowed.
 template <bool KC>
-__device__ inline u32x4_t a16_fetch8(const uint16_t* __restrict__ base, int line, int lines, int k0, int K, bool vec) {
+__device__ inline u32x4_t a16_fetch8(const uint16_t* __restrict__ base, int line, int lines, int k0, int K, size_t ld, bool vec) {
   u32x4_t v = {0u, 0u, 0u, 0u};
   if (line >= lines || k0 >= K) return v;
   if constexpr (KC) {
-    const uint16_t* p = base + (size_t)line * K + k0;
+    const uint16_t* p = base + (size_t)line * ld + k0;
     if (vec && k0 + 8 <= K) {
       __builtin_memcpy(&v, __builtin_assume_aligned(p, 16), 16);
       return v;
@@ -40,7 +40,7 @@ __device__ inline u32x4_t a16_fetch8(const uint16_t* __restrict__ base, int line
   } else {
     uint16_t t[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) t[e] = k0 + e < K ? base[(size_t)(k0 + e) * lines + line] : (uint16_t)0;
+    for (int e = 0; e < 8; e++) t[e] = k0 + e < K ? base[(size_t)(k0 + e) * ld + line] : (uint16_t)0;
     __builtin_memcpy(&v, t, 16);
   }
   return v;
@@ -60,8 +60,9 @@ __global__ void __launch_bounds__(A16_THREADS) mfma_acc16_kernel(GemmArgs<TYPES>
   const int M = g.M, N = g.N, K = g.K;
   const int tiles_n = (N + A16_BN - 1) / A16_BN;
   const int m0 = (int)(blockIdx.x / (unsigned)tiles_n) * A16_BM, n0 = (int)(blockIdx.x % (unsigned)tiles_n) * A16_BN;
-  const bool a_vec = A_KC && (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15u) == 0);
-  const bool b_vec = B_KC && (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15u) == 0);
+  const size_t lda = (size_t)g.lda, ldb = (size_t)g.ldb, ldc = (size_t)g.ldc, ldd = (size_t)g.ldd;
+  const bool a_vec = A_KC && (K % 8 == 0) && (lda % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15u) == 0);
+  const bool b_vec = B_KC && (K % 8 == 0) && (ldb % 8 == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15u) == 0);
 
   f32x16_t acc[FM][FN];
 #pragma unroll
@@ -77,8 +78,8 @@ __global__ void __launch_bounds__(A16_THREADS) mfma_acc16_kernel(GemmArgs<TYPES>
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const int p = tid + A16_THREADS * j, line = p >> 2, q = p & 3;
-      ra[j] = a16_fetch8<A_KC>(g.A, m0 + line, M, k0 + 8 * q, K, a_vec);
-      rb[j] = a16_fetch8<B_KC>(g.B, n0 + line, N, k0 + 8 * q, K, b_vec);
+      ra[j] = a16_fetch8<A_KC>(g.A, m0 + line, M, k0 + 8 * q, K, lda, a_vec);
+      rb[j] = a16_fetch8<B_KC>(g.B, n0 + line, N, k0 + 8 * q, K, ldb, b_vec);
     }
   };
   auto park = [&]() {
@@ -134,7 +135,8 @@ __global__ void __launch_bounds__(A16_THREADS) mfma_acc16_kernel(GemmArgs<TYPES>
 
   // acc[i][j][4 q + e] = D(m0 + 64 wm + 32 i + r32, n0 + 64 wn + 32 j + 8 q + 4 g2 + e)
   const bool use_c = g.beta != 0;
-  const bool vec = (N & 3) == 0 && ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & 7u) == 0;
+  const bool vec = (N & 3) == 0 && (ldd & 3) == 0 && (!use_c || (ldc & 3) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & 7u) == 0;
   static_for<FM>([&](auto i_c) {
     constexpr int I = decltype(i_c)::value;
     const int m = m0 + wm * 64 + I * 32 + r32;
@@ -144,20 +146,20 @@ __global__ void __launch_bounds__(A16_THREADS) mfma_acc16_kernel(GemmArgs<TYPES>
         constexpr int Q = decltype(q_c)::value;
         const int n = n0 + wn * 64 + J * 32 + Q * 8 + g2 * 4;
         if (m >= M || n >= N) return;
-        const size_t o = (size_t)m * N + n;
+        const size_t o = (size_t)m * ldd + n, oc = (size_t)m * ldc + n;
         if (vec) {   // N is a multiple of four: the lane's four columns exist together
           out_t cv[4] = {0, 0, 0, 0}, dv[4];
-          if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+          if (use_c) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
           dv[0] = epilogue<TYPES>(acc[I][J][4 * Q + 0], g.alpha, g.beta, &cv[0]);
           dv[1] = epilogue<TYPES>(acc[I][J][4 * Q + 1], g.alpha, g.beta, &cv[1]);
           dv[2] = epilogue<TYPES>(acc[I][J][4 * Q + 2], g.alpha, g.beta, &cv[2]);
           dv[3] = epilogue<TYPES>(acc[I][J][4 * Q + 3], g.alpha, g.beta, &cv[3]);
           __builtin_memcpy(g.D + o, dv, sizeof(dv));
         } else {
-          if (n + 0 < N) g.D[o + 0] = epilogue<TYPES>(acc[I][J][4 * Q + 0], g.alpha, g.beta, g.C + o + 0);
-          if (n + 1 < N) g.D[o + 1] = epilogue<TYPES>(acc[I][J][4 * Q + 1], g.alpha, g.beta, g.C + o + 1);
-          if (n + 2 < N) g.D[o + 2] = epilogue<TYPES>(acc[I][J][4 * Q + 2], g.alpha, g.beta, g.C + o + 2);
-          if (n + 3 < N) g.D[o + 3] = epilogue<TYPES>(acc[I][J][4 * Q + 3], g.alpha, g.beta, g.C + o + 3);
+          if (n + 0 < N) g.D[o + 0] = epilogue<TYPES>(acc[I][J][4 * Q + 0], g.alpha, g.beta, g.C + oc + 0);
+          if (n + 1 < N) g.D[o + 1] = epilogue<TYPES>(acc[I][J][4 * Q + 1], g.alpha, g.beta, g.C + oc + 1);
+          if (n + 2 < N) g.D[o + 2] = epilogue<TYPES>(acc[I][J][4 * Q + 2], g.alpha, g.beta, g.C + oc + 2);
+          if (n + 3 < N) g.D[o + 3] = epilogue<TYPES>(acc[I][J][4 * Q + 3], g.alpha, g.beta, g.C + oc + 3);
         }
       });
     });

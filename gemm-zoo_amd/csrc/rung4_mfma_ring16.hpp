@@ -212,6 +212,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr uint32_t COPY_BIAS = 4096;
   const int ci = lane >> 3, cs = lane & 7;
   const int N = g.N;
+  const size_t LDA = (size_t)g.lda * ES, LDB = (size_t)g.ldb * ES;   // bytes between the lines of A and of B
   // row-major B: group c carries K rows [HK c, HK c + HK) of B, BN elements each; a copy moves KRC whole K rows, the
   // lane at LDS position (row, slot) fetching the piece that belongs there (see ring16_row_swizzle)
   constexpr int KRC = 1024 / (BN * ES), LPR = 64 / KRC;
@@ -225,14 +226,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       // of B only, and those past the end are not stored)
       int r = 16 * (wave * A_PW + t) + 8 * par + ci;
       if constexpr (RAGGED) r = min(m0 + r, g.M - 1) - m0;
-      voff_a[par][t] = (uint32_t)((size_t)r * K * ES + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+      voff_a[par][t] = (uint32_t)((size_t)r * LDA + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
     }
     if constexpr (B_KC) {
 #pragma unroll
       for (int t = 0; t < B_PW; t++) {
         int r = 16 * (wave * B_PW + t) + 8 * par + ci;
         if constexpr (RAGGED) r = min(n0 + r, N - 1) - n0;
-        voff_b[par][t] = (uint32_t)((size_t)r * K * ES + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
+        voff_b[par][t] = (uint32_t)((size_t)r * LDB + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
       }
     }
   }
@@ -244,18 +245,18 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       const int kr = (wave * B_PW + t) * KRC + lane / LPR;   // K row within the group
       int piece = (lane % LPR) ^ ring16_row_swizzle<ES>(kr);
       if constexpr (RAGGED) piece = min(piece, last_piece);  // columns past the end: the last piece (not stored)
-      voff_b[0][t] = (uint32_t)(((size_t)kr * N + (size_t)(piece * EPV)) * ES) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
+      voff_b[0][t] = (uint32_t)((size_t)kr * LDB + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
     }
-    b_group_step = (size_t)HK * N * ES;
+    b_group_step = (size_t)HK * LDB;
   }
   // scalar bases of a tile: its first row of A (first column of a K-contiguous B) at the first K byte of this run; a
   // row-major B's first K row of the run at the tile's first column
   auto a_base_of = [&](int m_first) -> const char* {
-    return reinterpret_cast<const char*>(g.A) + (size_t)m_first * K * ES + k_byte0 - COPY_BIAS;
+    return reinterpret_cast<const char*>(g.A) + (size_t)m_first * LDA + k_byte0 - COPY_BIAS;
   };
   auto b_base_of = [&](int n_first) -> const char* {
-    if constexpr (B_KC) return reinterpret_cast<const char*>(g.B) + (size_t)n_first * K * ES + k_byte0 - COPY_BIAS;
-    else return reinterpret_cast<const char*>(g.B) + ((size_t)(2 * slab0) * HK * N + n_first) * ES - COPY_BIAS;
+    if constexpr (B_KC) return reinterpret_cast<const char*>(g.B) + (size_t)n_first * LDB + k_byte0 - COPY_BIAS;
+    else return reinterpret_cast<const char*>(g.B) + (size_t)(2 * slab0) * HK * LDB + (size_t)n_first * ES - COPY_BIAS;
   };
   // where copy group C of a tile starts, from the tile's bases
   auto a_group = [&](const char* a_tile, int c) -> const char* { return a_tile + (size_t)(c >> 1) * LINE; };
@@ -593,7 +594,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       gw.layoutA = g.layoutA; gw.layoutB = g.layoutB;
       gw.alpha = 1; gw.beta = 0;
       gw.store_hint = 0;
-      gw.ldb = BN; gw.ldd = BN;
+      gw.lda = K; gw.ldb = BN; gw.ldc = BN; gw.ldd = BN;
       store_accumulators_lds<WS_TYPES, WM / 32, WN / 32, false, 16>(gw, acc, wm * WM, wn * WN, lane,
                                                                     staging);
     } else {
@@ -637,21 +638,21 @@ __global__ void __launch_bounds__(256) streamk_fixup_kernel(GemmArgs<TYPES> g, i
   }
   const int m = tm * 256 + r, n = tn * 256 + c;
   if (m >= g.M || n >= g.N) return;
-  const size_t o = (size_t)m * g.ldd + n;
+  const size_t o = (size_t)m * g.ldd + n, oc = (size_t)m * g.ldc + n;
   const bool use_c = g.beta != 0;
   constexpr uintptr_t VEC_ALIGN = 4 * sizeof(out_t) - 1;
-  const bool vec = n + 4 <= g.N && (g.ldd & 3) == 0 &&
+  const bool vec = n + 4 <= g.N && (g.ldd & 3) == 0 && (!use_c || (g.ldc & 3) == 0) &&
                    ((reinterpret_cast<uintptr_t>(g.D) | (use_c ? reinterpret_cast<uintptr_t>(g.C) : 0)) & VEC_ALIGN) == 0;
   if (vec) {
     out_t cv[4] = {0, 0, 0, 0}, dv[4];
-    if (use_c) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+    if (use_c) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
 #pragma unroll
     for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, &cv[e]);
     __builtin_memcpy(g.D + o, dv, sizeof(dv));
   } else {
 #pragma unroll
     for (int e = 0; e < 4; e++)
-      if (n + e < g.N) g.D[o + e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, g.C + o + e);
+      if (n + e < g.N) g.D[o + e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, g.C + oc + e);
   }
 }
 

@@ -79,10 +79,10 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_reg_kernel(GemmArgs<TYPES> 
   // Rows past the end are clamped, not zeroed: an output element depends on one
   // row of A and one column of B only, and the clamped ones are never stored.
   const int n_ld = min(n_base + r16, g.N - 1);
-  const in_t* __restrict__ bp = g.B + (size_t)n_ld * K + grp * 16;
+  const in_t* __restrict__ bp = g.B + (size_t)n_ld * (size_t)g.ldb + grp * 16;
   const in_t* __restrict__ ap[MBLK];
 #pragma unroll
-  for (int i = 0; i < MBLK; i++) ap[i] = g.A + (size_t)min(16 * i + r16, g.M - 1) * K + grp * 16;
+  for (int i = 0; i < MBLK; i++) ap[i] = g.A + (size_t)min(16 * i + r16, g.M - 1) * (size_t)g.lda + grp * 16;
 
   sk_f32x4_t acc[MBLK];
 #pragma unroll
@@ -131,23 +131,23 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_reg_kernel(GemmArgs<TYPES> 
   // acc[i][v] = D(16 i + r16, n_base + 4 grp + v)
   const int N = g.N;
   const int n = n_base + 4 * grp;
-  const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
+  const bool vec_ok = (g.ldd % 4 == 0) && (g.beta == 0 || g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
                       (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
 #pragma unroll
   for (int i = 0; i < MBLK; i++) {
     const int m = 16 * i + r16;
     if (m >= g.M) continue;
-    const size_t o = (size_t)m * N + n;
+    const size_t o = (size_t)m * (size_t)g.ldd + n, oc = (size_t)m * (size_t)g.ldc + n;
     if (vec_ok && n + 3 < N) {
       out_t cv[4] = {0, 0, 0, 0}, dv[4];
-      if (g.beta != 0) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+      if (g.beta != 0) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
 #pragma unroll
       for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[i][e], g.alpha, g.beta, &cv[e]);
       __builtin_memcpy(g.D + o, dv, sizeof(dv));
     } else {
 #pragma unroll
       for (int e = 0; e < 4; e++)
-        if (n + e < N) g.D[o + e] = epilogue<TYPES>(acc[i][e], g.alpha, g.beta, g.C + o + e);
+        if (n + e < N) g.D[o + e] = epilogue<TYPES>(acc[i][e], g.alpha, g.beta, g.C + oc + e);
     }
   }
 }
@@ -215,10 +215,11 @@ __global__ void __launch_bounds__(KS * 64) skinny_dtl_kernel(GemmArgs<TYPES> g, 
   const int n_base = blockIdx.x * cols_per_wg;
   const int K = g.K, N = g.N, M = g.M;
   const uint32_t ring = lds_base + ks * (S * STAGE);
-  const size_t rowb = (size_t)K * 2;
+  const size_t rowb = (size_t)g.ldb * 2, rowb_a = (size_t)g.lda * 2;   // bytes between the columns of B and the rows of A
 
   // copy j moves rows 4j .. 4j+3 of the group: 16 lanes per row; the lane that fills position p of the LDS row
-  // fetches piece p ^ (row & 15) of the 256-byte chunk.  (n - n_base) * rowb < 2 * N * K < 2^32.
+  // fetches piece p ^ (row & 15) of the 256-byte chunk.  The offsets stay below 2^32: a work-group's columns times
+  // the pitch of B, the rows of A times its pitch (the launcher checks both).
   uint32_t voff[NCP];
 #pragma unroll
   for (int j = 0; j < NCP; j++) {
@@ -230,7 +231,7 @@ __global__ void __launch_bounds__(KS * 64) skinny_dtl_kernel(GemmArgs<TYPES> g, 
   const int r16 = lane & 15, grp = lane >> 4;
   uint32_t a_voff[MBLK];
 #pragma unroll
-  for (int mb = 0; mb < MBLK; mb++) a_voff[mb] = (uint32_t)((size_t)min(mb * 16 + r16, M - 1) * rowb) + grp * 16;
+  for (int mb = 0; mb < MBLK; mb++) a_voff[mb] = (uint32_t)((size_t)min(mb * 16 + r16, M - 1) * rowb_a) + grp * 16;
   const char* sa = reinterpret_cast<const char*>(g.A);
   // fragment of MFMA step t: row r16 of a column block, K piece 4t + grp
   uint32_t b_addr[4];
@@ -348,7 +349,7 @@ __global__ void __launch_bounds__(KS * 64) skinny_dtl_kernel(GemmArgs<TYPES> g, 
 
   // acc[mb][cb][v] = D(16 mb + r16, n_base + 16 cb + 4 grp + v)
   const int n_end = min(n_base + cols_per_wg, N);
-  const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
+  const bool vec_ok = (g.ldd % 4 == 0) && (g.beta == 0 || g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
                       (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
 #pragma unroll
   for (int mb = 0; mb < MBLK; mb++) {
@@ -357,17 +358,17 @@ __global__ void __launch_bounds__(KS * 64) skinny_dtl_kernel(GemmArgs<TYPES> g, 
 #pragma unroll
     for (int cb = 0; cb < CB; cb++) {
       const int n = n_base + cb * 16 + 4 * grp;
-      const size_t o = (size_t)m * N + n;
+      const size_t o = (size_t)m * (size_t)g.ldd + n, oc = (size_t)m * (size_t)g.ldc + n;
       if (vec_ok && n + 3 < n_end) {
         out_t cv[4] = {0, 0, 0, 0}, dv[4];
-        if (g.beta != 0) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+        if (g.beta != 0) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
 #pragma unroll
         for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[mb][cb][e], g.alpha, g.beta, &cv[e]);
         __builtin_memcpy(g.D + o, dv, sizeof(dv));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; e++)
-          if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(acc[mb][cb][e], g.alpha, g.beta, g.C + o + e);
+          if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(acc[mb][cb][e], g.alpha, g.beta, g.C + oc + e);
       }
     }
   }
@@ -400,7 +401,7 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
   const int K = g.K, N = g.N, M = g.M;
   const int n_base = blockIdx.x * cols_per_wg;
   const int n_end = min(n_base + cols_per_wg, N);
-  const size_t rowb = (size_t)K * 2;
+  const size_t rowb = (size_t)g.ldb * 2, rowb_a = (size_t)g.lda * 2;   // bytes between the columns of B and the rows of A
   const int nst = K / STREAM_TILE_K_STEP;
   const int rot = (int)(blockIdx.x % (unsigned)nst);
 
@@ -413,7 +414,7 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
 #pragma unroll
     for (int j = 0; j < NA; j++) {
       const int row = (p * NA + j) * 8 + row_in;
-      voffA[j] = (uint32_t)((size_t)min(row, M - 1) * rowb) + (pos ^ ((row >> 1) & 7)) * 16;
+      voffA[j] = (uint32_t)((size_t)min(row, M - 1) * rowb_a) + (pos ^ ((row >> 1) & 7)) * 16;
     }
 #pragma unroll
     for (int j = 0; j < NB; j++) {
@@ -517,7 +518,7 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
         for (int e = 0; e < 16; e++) acc[r][e] += red[((((q - 1) * 2 * NRG + tile) * NRB + r) * 16 + e) * 64 + lane];
   }
 
-  const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
+  const bool vec_ok = (g.ldd % 4 == 0) && (g.beta == 0 || g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
                       (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
 #pragma unroll
   for (int r = 0; r < NRB; r++) {
@@ -526,17 +527,17 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       const int n = n_base + cbw * 32 + q * 8 + g2 * 4;
-      const size_t o = (size_t)m * N + n;
+      const size_t o = (size_t)m * (size_t)g.ldd + n, oc = (size_t)m * (size_t)g.ldc + n;
       if (vec_ok && n + 3 < n_end) {
         out_t cv[4] = {0, 0, 0, 0}, dv[4];
-        if (g.beta != 0) __builtin_memcpy(cv, g.C + o, sizeof(cv));
+        if (g.beta != 0) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
 #pragma unroll
         for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(acc[r][4 * q + e], g.alpha, g.beta, &cv[e]);
         __builtin_memcpy(g.D + o, dv, sizeof(dv));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; e++)
-          if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(acc[r][4 * q + e], g.alpha, g.beta, g.C + o + e);
+          if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(acc[r][4 * q + e], g.alpha, g.beta, g.C + oc + e);
       }
     }
   }
@@ -557,8 +558,9 @@ template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hi
                 SKINNY_MAX_M, SKINNY_K_STEP, g.M, g.K);
       return GZ_ERR_UNSUPPORTED;
     }
-    if ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15u) {
-      set_error("skinny rung needs 16-byte aligned A and B");
+    if (((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15u) || !skinny_lines_ok(g.lda, g.ldb)) {
+      set_error("skinny rung needs 16-byte aligned A and B and leading dimensions that are multiples of 8 elements "
+                "(lda=%lld ldb=%lld)", (long long)g.lda, (long long)g.ldb);
       return GZ_ERR_UNSUPPORTED;
     }
     const SkinnyCfg c = skinny_resolve(g.M, g.N, g.K, device_compute_units());

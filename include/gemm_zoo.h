@@ -3,11 +3,15 @@
  *
  * D = alpha * (A x B) + beta * C   with A: M x K, B: K x N, C and D: M x N.
  *
- * All matrix pointers are DEVICE pointers owned by the caller, packed (the
- * leading dimension equals the contiguous extent).  C and D are always
- * row-major.  A and B carry a layout flag each.  When beta == 0, C is never
- * read and may be NULL.  D must not overlap A or B.  Calls are asynchronous on
- * `stream` (a hipStream_t, NULL = the default stream); the caller synchronises.
+ * All matrix pointers are DEVICE pointers owned by the caller.  The typed entry
+ * points and gz_gemm take packed matrices (the leading dimension equals the
+ * contiguous extent); gz_gemm_ld takes the four leading dimensions.  C and D are
+ * always row-major.  A and B carry a layout flag each.  When beta == 0, C is
+ * never read and may be NULL.  D must not overlap A or B.  Calls are
+ * asynchronous on `stream` (a hipStream_t, NULL = the default stream); the
+ * caller synchronises.  M, N, K and the leading dimensions stay below 2^31; the
+ * matrices themselves may hold 2^31 elements and more (the reference indexes
+ * with std::size_t, nvidia/utils/benchmark.cuh:17, nvidia/kernels/naive_gemm.cuh:8).
  *
  * Every function returns a gz_status; nothing exits the process or throws.
  * gz_last_error() gives the message of the calling thread's last failure.
@@ -188,6 +192,17 @@ int gz_gemm_f16f16f16_acc16(const uint16_t* A, const uint16_t* B, const uint16_t
 int gz_gemm(int types, const void* A, const void* B, const void* C, void* D,
             int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
             double alpha, double beta, int rung, int variant, gz_stream stream);
+
+/* gz_gemm on matrices with leading dimensions, in elements, as nvidia::kernels::generic_gemm takes them
+ * (nvidia/kernels/generic_gemm.cuh:6-8; its functor passes the packed values, nvidia/kernel_functors/generic_gemm.cuh:30-32):
+ * lda between consecutive rows of a row-major A (at least K) or columns of a column-major one (at least M), ldb between
+ * the K rows of a row-major B (at least N) or the columns of a column-major one (at least K), ldc / ldd between the rows
+ * of C / D (at least N).  0 stands for the packed value.  Every rung takes them; the direct-to-LDS kernels of the MFMA
+ * rung and the weight-streaming rung need leading dimensions that are whole 16-byte pieces (the launcher's choice falls
+ * back to the register-staged kernels otherwise, an explicit GZ_RUNG_SKINNY returns GZ_ERR_UNSUPPORTED).            */
+int gz_gemm_ld(int types, const void* A, int64_t lda, const void* B, int64_t ldb, const void* C, int64_t ldc,
+               void* D, int64_t ldd, int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
+               double alpha, double beta, int rung, int variant, gz_stream stream);
 
 /* gz_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and the same results,

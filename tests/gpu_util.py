@@ -66,3 +66,46 @@ def assert_within(types, got, truth_f64, what=""):
     worst = float((err / np.maximum(bound, 1e-300)).max()) if err.size else 0.0
     assert worst <= 1.0, f"{what}: error is {worst:.3f} x the allowed {tol} relative bound"
     return worst * tol
+
+
+def run_gemm_ld(types, a, b, c, m, n, k, la, lb, alpha, beta, rung, variant=0, pads=(0, 0, 0, 0), misalign=0):
+    """gz_gemm_ld on sub-matrix views: every operand sits in a wider allocation whose leading dimension is its packed
+    one plus pads[i] elements, the padding filled with a pattern that is a NaN for the float types and a large value
+    for int8, so that a kernel that reads across a line's end shows.  a, b, c are the packed host arrays (a: m x k or
+    k x m as its layout says, flat is fine).  Returns D (m x n) and checks that neither the padding of D nor the
+    words around it were written."""
+    def lines(layout_rows_major, rows, cols):   # (number of lines, line length)
+        return (rows, cols) if layout_rows_major else (cols, rows)
+
+    def widen(x, nlines, length, pad):
+        x = np.asarray(x).reshape(nlines, length)
+        big = np.empty((nlines, length + pad), dtype=x.dtype)
+        # NaN patterns of bf16 / fp16 (0x7fc1), e4m3 / e5m2 (0x7f), fp32; large values for the integer types
+        big[...] = {np.dtype(np.uint16): 0x7FC1, np.dtype(np.uint8): 0x7F, np.dtype(np.int8): 127,
+                    np.dtype(np.int32): 0x5A5A5A5A, np.dtype(np.float32): np.nan}[x.dtype]
+        big[:, :length] = x
+        return big
+
+    an, al = lines(la == O.ROW, m, k)
+    bn, bl = lines(lb == O.ROW, k, n)
+    pa, pb, pc, pd = pads
+    abig = widen(a, an, al, pa)
+    bbig = widen(b, bn, bl, pb)
+    da, db = up(abig.reshape(-1), misalign), up(bbig.reshape(-1), misalign)
+    dc = None
+    if c is not None:
+        cbig = widen(c, m, n, pc)
+        dc = up(cbig.reshape(-1), misalign)
+    sentinel = 0x5A5A if O.OUT_DTYPE[types] == np.uint16 else 0x5A5A5A5A
+    guard = 64
+    ldd = n + pd
+    full = torch.full((m * ldd + 2 * guard,), sentinel, dtype=out_torch_dtype(types), device=dev())
+    dd = full[guard:guard + m * ldd]
+    capi.gemm_ld(types, da, al + pa, db, bl + pb, dc, n + pc, dd, ldd, m, n, k, la, lb, alpha, beta, rung, variant,
+                 torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    host = full.cpu()
+    assert (host[:guard] == sentinel).all() and (host[guard + m * ldd:] == sentinel).all(), "wrote outside D"
+    body = host[guard:guard + m * ldd].reshape(m, ldd)
+    assert (body[:, n:] == sentinel).all(), "wrote into the padding between the rows of D"
+    return np.ascontiguousarray(body[:, :n].numpy()).view(O.OUT_DTYPE[types]).reshape(m, n)

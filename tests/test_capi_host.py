@@ -37,7 +37,7 @@ def test_version_and_names(capi):
 @pytest.mark.parametrize("kwargs,status", [
     (dict(types=9), 1), (dict(m=-1), 1), (dict(k=-5), 1), (dict(layout_a=2), 1), (dict(layout_b=-1), 1),
     (dict(rung=6), 1), (dict(rung=-2), 1), (dict(variant=-1), 1),
-    (dict(m=1 << 20, k=1 << 20), 2),            # 2^40 elements
+    (dict(m=1 << 31), 2),                       # an extent of 2^31 (2^40 elements with smaller extents are fine)
     (dict(rung=4, variant=99), 2),
     (dict(rung=0, variant=1), 2),
     (dict(types=0, rung=5), 2),                 # no int8 streaming kernel
@@ -206,3 +206,27 @@ def test_tile_choice_on_the_register_staged_kernel(capi):
     assert tile(capi.F32F32F32, 3000, 3000, 1000, 0, 0)[:2] == (128, 128)
     assert tile(capi.F32F32F32, 4096, 4096, 4000, 0, 1)[:2] == (256, 256)
     assert tile(capi.F32F32F32, 1000, 8000, 4000, 0, 1)[:2] == (256, 128)
+
+
+def test_leading_dimension_arguments(capi):
+    """gz_gemm_ld checks its leading dimensions before anything touches a device: each at least the extent of a line,
+    none negative, none of 2^31 or more; and extents of 2^31 are refused while element counts beyond 2^31 are not an
+    argument error."""
+    ld = capi.lib.gz_gemm_ld
+    base = dict(types=1, a=64, lda=0, b=64, ldb=0, c=0, ldc=0, d=64, ldd=0, m=4, n=6, k=8, la=0, lb=1, alpha=1.0, beta=0.0,
+                rung=-1, variant=0, stream=None)
+
+    def call(**kw):
+        v = dict(base, **kw)
+        return ld(v["types"], v["a"], v["lda"], v["b"], v["ldb"], v["c"], v["ldc"], v["d"], v["ldd"], v["m"], v["n"], v["k"],
+                  v["la"], v["lb"], v["alpha"], v["beta"], v["rung"], v["variant"], v["stream"])
+    assert call(lda=7) == capi.ERR_BAD_ARG and "lda" in capi.last_error()            # row-major A: at least K
+    assert call(la=1, lda=3) == capi.ERR_BAD_ARG                                      # column-major A: at least M
+    assert call(ldb=7) == capi.ERR_BAD_ARG and call(lb=0, ldb=5) == capi.ERR_BAD_ARG  # column-major B: K; row-major: N
+    assert call(ldc=5) == capi.ERR_BAD_ARG and call(ldd=5) == capi.ERR_BAD_ARG
+    assert call(lda=-1) == capi.ERR_BAD_ARG
+    assert call(lda=1 << 31) == capi.ERR_UNSUPPORTED
+    assert call(m=1 << 31) == capi.ERR_UNSUPPORTED
+    # 65536 x 65536 x 32768 holds 2^31 and 2^32 elements per matrix: planned like any other problem
+    p = capi.plan(capi.S8S8S32, 65536, 65536, 32768, 0, 1)
+    assert p.rung == capi.RUNG_MFMA and (p.tile_m, p.tile_n) == (256, 256)

@@ -281,3 +281,63 @@ def test_sign_of_zero_survives_the_epilogue(G, types):
     assert (ref.view(np.uint8).reshape(m * n, -1)[:, -1] == 0x80).all()
     for rung in VALU_RUNGS + (MFMA,):
         assert np.array_equal(G.run_gemm(types, z, b, c, m, n, k, O.ROW, O.COL, -1, 0, rung), ref), (types, rung)
+
+
+def ld_pads(types):
+    """Leading-dimension paddings in elements: whole 16-byte pieces on every operand (the direct-to-LDS kernels keep
+    working), odd ones (every kernel that needs aligned lines has to step aside), and a mix."""
+    piece_in = 16 // np.dtype(O.IN_DTYPE[types]).itemsize
+    piece_out = 16 // np.dtype(O.OUT_DTYPE[types]).itemsize
+    return [(piece_in, 2 * piece_in, piece_out, 3 * piece_out), (3, 1, 5, 7), (piece_in, 0, 1, piece_out)]
+
+
+@pytest.mark.parametrize("types", ALL_TYPES)
+@pytest.mark.parametrize("rung", (-1,) + VALU_RUNGS + (MFMA,))
+def test_leading_dimensions_every_rung(G, types, rung):
+    """gz_gemm_ld on sub-matrix views (nvidia/kernels/generic_gemm.cuh:6-8 takes lda, ldb, ldc, ldd): A, B, C and D
+    each inside a wider allocation, paddings aligned and not, every layout pair; bit-exact against the oracle on the
+    packed copies of the same sub-matrices, the paddings of D untouched."""
+    shapes = [(65, 63, 33), (256, 256, 256), (300, 200, 128)]
+    for (la, lb), (m, n, k), pads in itertools.product(LAYOUTS, shapes, ld_pads(types)):
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=m + n + k + pads[0])
+        print("case", types, rung, la, lb, m, n, k, pads, flush=True)
+        got = G.run_gemm_ld(types, a, b, c, m, n, k, la, lb, 2, -1, rung, 0, pads)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 2, -1)), (types, rung, la, lb, m, n, k, pads)
+
+
+@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.F16F16F16, O.E4M3E4M3F16))
+def test_leading_dimensions_on_the_direct_kernels(G, types):
+    """Whole 256 x 256 tiles with leading dimensions of whole 16-byte pieces stay on the ring kernel (variants 5, 6:
+    both layouts of B, stream-K with variant 7) and on the compiler-scheduled direct-to-LDS kernels (variants 2, 3);
+    ragged M and N with them on the ring kernel's ragged instance; odd paddings send the same calls to the
+    register-staged kernel.  Bit-exact either way."""
+    slab = 128 // np.dtype(O.IN_DTYPE[types]).itemsize
+    piece_in = 16 // np.dtype(O.IN_DTYPE[types]).itemsize
+    piece_out = 16 // np.dtype(O.OUT_DTYPE[types]).itemsize
+    cases = [(512, 256, 6 * slab), (300, 520, 3 * slab)]
+    pad_sets = [(2 * piece_in, piece_in, piece_out, 2 * piece_out), (piece_in, piece_in, 1, 1), (1, 3, piece_out, piece_out)]
+    variants = (2, 3, 5, 6) + ((7,) if types in (O.S8S8S32, O.BF16BF16F32, O.F16F16F16) else ())
+    for variant, lb, (m, n, k), pads in itertools.product(variants, (O.COL, O.ROW), cases, pad_sets):
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=variant + k)
+        print("case", types, variant, lb, m, n, k, pads, flush=True)
+        got = G.run_gemm_ld(types, a, b, c, m, n, k, O.ROW, lb, 1, 1, MFMA, variant, pads)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, lb, 1, 1)), (types, variant, lb, m, n, k, pads)
+
+
+@pytest.mark.parametrize("types", SKINNY_TYPES)
+def test_leading_dimensions_on_the_streaming_rung(G, types):
+    """The weight-streaming kernels take leading dimensions of whole 16-byte pieces; others are refused by the rung
+    itself and served by the tiled rung under the launcher's choice."""
+    for (m, n, k), pads in itertools.product([(1, 520, 256), (8, 512, 192), (24, 300, 512), (100, 448, 1024)],
+                                             [(8, 16, 4, 8), (16, 8, 1, 3)]):
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=m + n)
+        ref = O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1)
+        for rung in (SKINNY, -1):
+            print("case", types, rung, m, n, k, pads, flush=True)
+            assert np.array_equal(G.run_gemm_ld(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1, rung, 0, pads), ref), (m, n, k, pads, rung)
+    a, b, c = O.make_inputs(types, 8, 512, 256, kind=O.FILL_SMALL_INT, seed=1)
+    with pytest.raises(G.capi.GzError) as e:
+        G.run_gemm_ld(types, a, b, c, 8, 512, 256, O.ROW, O.COL, 1, 1, SKINNY, 0, (3, 8, 0, 0))
+    assert e.value.status == G.capi.ERR_UNSUPPORTED
+    assert np.array_equal(G.run_gemm_ld(types, a, b, c, 8, 512, 256, O.ROW, O.COL, 1, 1, -1, 0, (3, 8, 0, 0)),
+                          O.gemm(types, a, b, c, 8, 512, 256, O.ROW, O.COL, 1, 1))
