@@ -26,6 +26,7 @@ FILL_INT8_UNIFORM, FILL_NORMAL, FILL_UNIFORM_PM1, FILL_SMALL_INT = 0, 1, 2, 3
 # decomposition, and the ring kernel with one work-group per tile instead of one per compute unit
 MFMA_256_W4, MFMA_256_W8, MFMA_128, MFMA_256X128 = 1, 2, 3, 4
 MFMA_RING_W4, MFMA_RING_W8, MFMA_STREAMK_W4, MFMA_STREAMK_W8, MFMA_RING_W4_PER_TILE, MFMA_RING_W8_PER_TILE = 5, 6, 7, 8, 9, 10
+MFMA_RING_128 = 11
 
 TYPES_NAMES = {S8S8S32: "s8s8s32", BF16BF16F32: "bf16bf16f32", BF16BF16BF16: "bf16bf16bf16", F16F16F16: "f16f16f16",
                F32F32F32: "f32f32f32", E4M3E4M3F16: "e4m3e4m3f16", E5M2E5M2F16: "e5m2e5m2f16",

@@ -33,11 +33,12 @@ static const MfmaCfg kMfmaCfgs[] = {
     {8, 256, 256, 2, 4, 1, true},    // variant 6, the same
     {9, 256, 256, 2, 2, 2, false},   // variant 5 with one work-group per tile (for comparisons with the persistent launch)
     {10, 256, 256, 2, 4, 2, false},  // variant 6, the same
+    {11, 128, 128, 2, 2, 2, false},  // tile of variant 3 on the ring kernel, two work-groups per compute unit
 };
 constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
 // positions in the table
 enum { MFMA_CFG_256_W4 = 0, MFMA_CFG_256_W8 = 1, MFMA_CFG_128 = 2, MFMA_CFG_256x128 = 3, MFMA_CFG_RING_W4 = 4,
-       MFMA_CFG_RING_W8 = 5 };
+       MFMA_CFG_RING_W8 = 5, MFMA_CFG_RING_128 = 10 };
 enum { MFMA_VARIANT_RING_W4 = 5, MFMA_VARIANT_RING_W8 = 6, MFMA_VARIANT_STREAMK_W4 = 7, MFMA_VARIANT_STREAMK_W8 = 8 };
 
 // the most any kernel of the configuration asks for: the ring kernel keeps five buffers of half a slab each
@@ -113,7 +114,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
   // candidates: 256x256 (on the ring kernel where the types and the layout of A allow it), 256x128, 128x128
   const bool ring_ok = a_rows && types != GZ_F32F32F32;
-  const int cand[3] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128, MFMA_CFG_128};
+  const bool ring128_ok = ring_ok && types != GZ_E4M3E4M3F16 && types != GZ_E5M2E5M2F16;
+  const int cand[3] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,
+                       ring128_ok ? MFMA_CFG_RING_128 : MFMA_CFG_128};
   double best = 0;
   int pick = cand[0];
   for (int i = 0; i < 3; i++) {
@@ -149,10 +152,20 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // costs: 256 x 128 half a round per round of its own, 128 x 128 its tiles over four per compute unit (measured,
     // in rounds of 256 x 256, 128 x 128 / 256 x 128: 6000 x 6000 x 3000 2.56 / 2.69 against 3.19; 3000 x 3000 x 1000
     // 0.79 / 1.03 against 1; 5000^3 1.99 / 2.13 against 2.13; 4096 x 4096 x 4000 1.13 / 1.02 against 1).
+    // 128 x 128 tiles on the ring kernel, two work-groups per compute unit: a "double round" of up to 2 x CUs tiles
+    // costs 0.36 + 0.15 tiles / CUs of a round of 256 x 256 tiles (bf16 -> f32 cubes, us: 1024 13.5, 1536 21.8, 2048
+    // 27.8, 2560 39.0, 3072 74.7 against rounds of 34, 44, 55, 65, 76); the register-staged kernel of the same tile,
+    // which the launcher keeps for a K-contiguous B while every work-group has a compute unit to itself, within 0.04
+    // of that.
+    if (i == 2 && direct && ring128_ok) {
+      const long long full2 = tiles / (2LL * num_cus), rem2 = tiles % (2LL * num_cus);
+      shape_cost = 0.66 * full2 + (rem2 ? 0.36 + 0.15 * (double)rem2 / num_cus : 0.0);
+    }
     if (f32 && i == 1) shape_cost = 0.52 * rounds;
     if (f32 && i == 2) shape_cost = 0.10 + 1.15 * (double)tiles / (4.0 * num_cus);
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
-    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : 1.15) : 1.0;
+    // (the ring kernel takes a row-major B through the transposing reads at no cost to speak of, on either tile)
+    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : ring128_ok ? 1.0 : 1.15) : 1.0;
     // What the register-staged kernel costs over a direct-to-LDS one on the same tile (4096 x 4096 x 4000 against
     // 4096^3, us: bf16 256 x 256 on eight waves 121 / 100, 128 x 128 155 against an estimated 150; int8 73 / 58 and
     // 98 / 87; fp8, four waves, 81 / 52 and 92 / 90).  On 128 x 128 tiles it grows with the rounds beyond four (twice
@@ -171,6 +184,14 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     }
   }
   *out = kMfmaCfgs[pick];
+  if (pick == MFMA_CFG_RING_128) {
+    // A K-contiguous B while every work-group has a compute unit to itself: the register-staged kernel, whose plain
+    // loads get a little more out of a lone work-group's path to the L2 (us, ring / register-staged, bf16 cubes:
+    // 1024 13.5 / 13.3, 1536 21.8 / 19.3, 2048 27.8 / 25.6; two per compute unit: 2560 39.0 / 44.5).  A row-major B
+    // always the ring (1024 13.8 / 18.6, 2048 27.9 / 39.9; int8 1024^3 9.3 / 10.9).
+    const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
+    if (b_cols && tiles <= num_cus) *out = kMfmaCfgs[MFMA_CFG_128];
+  }
   if (pick == MFMA_CFG_RING_W4) {
     // Waves per 256 x 256 tile on the ring kernel.
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
@@ -433,7 +454,7 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
   double est_rows = 0, est_cols = 0, best = single_rounds;
   if (mfma_resolve_split(types, M, N, K, layoutA, layoutB, num_cus, &sp, &est_rows) && est_rows < best) best = est_rows;
   if (mfma_resolve_colsplit(types, M, N, K, layoutA, layoutB, num_cus, &cs, &est_cols) && est_cols < best) best = est_cols;
-  return out->estimate_us < 0.95 * best * round_us;
+  return out->estimate_us < 0.99 * best * round_us;
 }
 
 // Work-groups of a launch of whole tiles on the ring kernel: past one round of the compute units the kernel is

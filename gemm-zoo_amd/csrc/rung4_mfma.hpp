@@ -1050,6 +1050,13 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
         else GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
       }
     }
+    // the same kernel on whole 128 x 128 tiles (int8 and the 16-bit types), one work-group per tile, two per compute unit
+    if constexpr (BM == 128 && BN == 128 && WAVES_M == 2 && WAVES_N == 2 && !is_fp8(TYPES)) {
+      if (ring && akc && !edge) {
+        if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});
+        else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
+      }
+    }
     if (!edge && akc && bkc) {  // whole tiles, both operands K-contiguous
       // The compiler-scheduled direct-to-LDS kernel is kept for the eight-wave 256x256 tile only: with four waves the
       // register-staged kernel below, whose loads and LDS stores are spread between the MFMAs, measured faster on
@@ -1292,6 +1299,7 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
     case 6: case 8: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 1, s);
     case 9: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s);
     case 10: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s);
+    case 11: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 2, s);
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);

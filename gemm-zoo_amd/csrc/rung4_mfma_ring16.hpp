@@ -113,12 +113,18 @@ constexpr size_t STREAMK_SLOT_ELEMS = 256 * 256;
 // transposing read takes, per 16 lanes, a block of 4 (16-bit) or 8 (int8) K rows, and the four lane groups of a
 // fragment take blocks 8 (16) rows apart: the first term spreads the rows of a block over the banks, the second
 // the two blocks that one half of the wave reads in the same cycle.
-template <int ES> __host__ __device__ constexpr int ring16_row_swizzle(int r) {
-  return ES == 2 ? (((r & 3) << 2) ^ (((r >> 3) & 1) << 1)) : (((r & 7) << 1) ^ ((r >> 4) & 1));
+// (Rows of 128 bytes - int8 with a 128-column tile - hold eight pieces, and consecutive rows already lie in different
+// halves of the 64 banks: the row's lowest bit stays out of the swizzle, which then fits three bits.)
+template <int ES, int ROW_BYTES> __host__ __device__ constexpr int ring16_row_swizzle(int r) {
+  static_assert(ROW_BYTES >= 256 || (ES == 1 && ROW_BYTES == 128), "a K row of at least sixteen pieces, or eight of int8");
+  return ES == 2 ? (((r & 3) << 2) ^ (((r >> 3) & 1) << 1))
+                 : ROW_BYTES >= 256 ? (((r & 7) << 1) ^ ((r >> 4) & 1)) : ((((r >> 1) & 3) << 1) ^ ((r >> 4) & 1));
 }
 
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool RAGGED = false, bool STREAMK = false, bool B_KC = true>
-__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
+// (second launch bound: waves per SIMD the registers must leave room for - the 128 x 128 tile, whose five buffers are
+// half the LDS, runs two work-groups per compute unit)
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128) ? 2 : (WAVES_M * WAVES_N) / 4)
     mfma_ring16_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n, StreamK sk) {
   using T = Traits<TYPES>;
   using in_t = typename T::in_t;
@@ -141,9 +147,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (8 rows) per wave and group
   constexpr int NCP = A_PW + B_PW;
   static_assert(TYPES != GZ_F32F32F32, "8- and 16-bit operands");
-  // (the kernel also compiles for a 128 x 128 tile on four waves, but its results there are wrong and it reads
-  // outside the operands: the split of a slab's rows over the copy groups is written for this tile only)
-  static_assert(BM == 256 && BN == 256, "written and tested for the 256 x 256 tile");
+  static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && NW == 4 && !F8 && !STREAMK),
+                "the 256 x 256 tile, or the 128 x 128 tile on four waves for int8 and the 16-bit types");
   static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile rows must divide over the waves");
   static_assert(A_PW <= 8 && B_PW <= 8 && A_PW % 2 == 0 && B_PW % 2 == 0, "a copy group must fit the immediate offset range");
   static_assert(NCP == 8 || NCP == 4, "the vmcnt immediates below are written out for 8 or 4 copies per wave and group");
@@ -243,7 +248,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 #pragma unroll
     for (int t = 0; t < B_PW; t++) {
       const int kr = (wave * B_PW + t) * KRC + lane / LPR;   // K row within the group
-      int piece = (lane % LPR) ^ ring16_row_swizzle<ES>(kr);
+      int piece = (lane % LPR) ^ ring16_row_swizzle<ES, BN * ES>(kr);
       if constexpr (RAGGED) piece = min(piece, last_piece);  // columns past the end: the last piece (not stored)
       voff_b[0][t] = (uint32_t)((size_t)kr * LDB + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
     }
@@ -307,7 +312,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     const int i16 = lane & 15, ti = i16 / TR_LPR;
     const int n_sub = (i16 % TR_LPR) * (8 / ES);
     const int krow = quarter * (2 * 16 / TR_LPR) + ti;
-    const int f = ring16_row_swizzle<ES>(krow);           // the same for the second half: its rows differ in bit 2 (3) only
+    const int f = ring16_row_swizzle<ES, BN * ES>(krow);           // the same for the second half: its rows differ in bit 2 (3) only
     // Block j of the wave starts 16 j columns further, i.e. 16 j / EPV pieces: j pieces for 8-bit elements, 2 j for
     // 16-bit ones.  Those are bits of the piece number that nothing else of it touches (the wave's first column is
     // a multiple of 64, the lane's column within a block less than 16), the swizzle is an exclusive-or on the piece

@@ -126,26 +126,28 @@ def test_c5_skinny_bf16(G, m):
 
 
 @pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16])
-@pytest.mark.parametrize("shape,tile", [((4096, 4096, 512), (256, 256)), ((2048, 4096, 1024), (256, 128)),
-                                        ((512, 384, 256), (128, 128)), ((256, 128, 128), (128, 128))])
-def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile):
+@pytest.mark.parametrize("shape,tile,variant", [((4096, 4096, 512), (256, 256), 0), ((2048, 4096, 1024), (128, 128), 0),
+                                                ((2048, 4096, 1024), (256, 128), 4), ((512, 384, 256), (128, 128), 0),
+                                                ((256, 128, 128), (128, 128), 0), ((512, 384, 256), (128, 128), 3)])
+def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile, variant):
     """Row-major A and B (every driver of the reference).  The first shape gives each compute unit a whole 256x256
-    tile (hand-scheduled kernel, transposing LDS reads for B), the others take the smaller tiles without predication
-    (256x128: register-staged kernel; 128x128: direct-to-LDS kernel with transposing LDS reads)."""
+    tile (hand-scheduled ring kernel, transposing LDS reads for B), the others take the smaller tiles without
+    predication: 128x128 on the same ring kernel with two work-groups per compute unit (the launcher's choice), 256x128
+    on the register-staged kernel and 128x128 on the compiler-scheduled direct-to-LDS kernel (variants 4 and 3)."""
     m, n, k = shape
-    p = G.capi.plan(types, m, n, k, O.ROW, O.ROW)
+    p = G.capi.plan(types, m, n, k, O.ROW, O.ROW, 4 if variant else -1, variant)
     assert p.rung == 4 and m % p.tile_m == 0 and n % p.tile_n == 0          # whole tiles: no predicated kernel
     assert (p.tile_m, p.tile_n) == tile
     kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT   # exact partial sums in any order
     a, b, ha, hb = device_inputs(G, types, m, n, k, kind, 77)
     hc = O.fill(m * n, O.OUT_DT[types], O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT, 1.0, 79)
-    got = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, O.ROW, 1, 1, -1)
+    got = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, O.ROW, 1, 1, 4 if variant else -1, variant)
     rows = (0, m) if m <= 512 else (m - 24, m)
     ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, O.ROW, 1, 1, rows=rows)
     assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]])
     if types != O.S8S8S32:  # N(0,1) operands against fp64 truth
         a, b, ha, hb = device_inputs(G, types, m, n, k, O.FILL_NORMAL, 78)
-        got = G.run_gemm(types, ha, hb, None, m, n, k, O.ROW, O.ROW, 1, 0, -1)
+        got = G.run_gemm(types, ha, hb, None, m, n, k, O.ROW, O.ROW, 1, 0, 4 if variant else -1, variant)
         truth, _ = O.gemm_f64(types, ha, hb, None, m, n, k, O.ROW, O.ROW, 1, 0, rows=(8, 24))
         G.assert_within(types, got[8:24], truth, f"row/row {shape}")
 

@@ -20,11 +20,13 @@ BIN = ROOT / "gemm-zoo_amd" / "bench" / "bin"
 
 # driver -> (lines expected, largest dimension let through)
 DRIVERS = {
-    "bench_bf16_mma_gemm": (4, 2048),            # 256 .. 2048 of the reference's list; the 4096 / 8192 headline sizes are cut
-    "bench_fp16_mma_gemm": (4, 2048),            # the same list; 4095 x 4097 x 1023 is cut by its N
-    "bench_xe_gemm_s8_s8_s32_m8k16": (2, 2048),  # 1024, 2048
+    # 256 .. 4096 of the reference's list (row-major B, alpha = beta = 1) and the 4096^3 headline (column-major B):
+    # the functor constructors plan, launch and verify the 256 x 256 ring kernel from C++; 8192^3 is cut
+    "bench_bf16_mma_gemm": (6, 4096),
+    "bench_fp16_mma_gemm": (6, 4097),            # the same list and the ragged 4095 x 4097 x 1023
+    "bench_xe_gemm_s8_s8_s32_m8k16": (3, 4096),  # 1024, 2048, 4096
     "bench_ladder": (18, 2048),                  # three type bundles x six rungs at 2048^3
-    "bench_fp8_mma_gemm": (10, 4096),            # e4m3 and e5m2, 256 .. 4096: the last one runs the 256 x 256 ring kernel
+    "bench_fp8_mma_gemm": (10, 4096),            # e4m3 and e5m2, 256 .. 4096
 }
 
 
@@ -34,7 +36,7 @@ def test_cpp_driver_runs_and_verifies(driver):
     if not exe.exists():
         pytest.fail(f"{exe} is not built (python gemm-zoo_amd/build.py builds the drivers)")
     want, max_dim = DRIVERS[driver]
-    env = dict(os.environ, GZ_BENCH_MAX_DIM=str(max_dim), GZ_BENCH_REPS="3")
+    env = dict(os.environ, GZ_BENCH_MAX_DIM=str(max_dim), GZ_BENCH_REPS="2")
     print("running", driver, flush=True)
     proc = subprocess.run([str(exe)], env=env, capture_output=True, text=True, timeout=240)
     out = proc.stdout + proc.stderr
