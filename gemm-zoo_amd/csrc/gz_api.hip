@@ -422,6 +422,23 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         plan->grid = (int64_t)ceil_div(m, 128) * ceil_div(n, 128);
         return GZ_OK;
       }
+      if (MfmaCfg ct; mfma_transposed_ring(types, m, n, k, layoutA, layoutB, variant, num_cus, &ct)) {
+        // column-major A and B: the ring kernel on the transposed problem (as launch_mfma, aligned operands assumed);
+        // the configuration's rows run along N there
+        plan->variant = ct.id;
+        plan->tile_m = ct.bn; plan->tile_n = ct.bm; plan->tile_k = MFMA_SLAB_BYTES / es;
+        plan->wave_m = ct.bn / ct.waves_m; plan->wave_n = ct.bm / ct.waves_n;
+        plan->threads = ct.waves_m * ct.waves_n * 64;
+        plan->lds_bytes = mfma_lds_bytes(ct);
+        plan->grid = (int64_t)ceil_div(n, ct.bm) * ceil_div(m, ct.bn);
+        if (ct.ring == 1 && mfma_shape_class(ct, es, n, m, k, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE)
+          plan->grid = mfma_persistent_grid(plan->grid, num_cus);
+        if (plan->lds_bytes > lds_per_cu) {
+          set_error("mfma variant %d needs %d bytes of LDS, device has %d", ct.id, plan->lds_bytes, lds_per_cu);
+          return GZ_ERR_UNSUPPORTED;
+        }
+        return GZ_OK;
+      }
       if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && k > 0) {   // as launch_mfma, aligned operands assumed
         StreamKPlan skp;
         const MfmaCfg* forced = variant == 0 ? nullptr : &kMfmaCfgs[variant - 1];

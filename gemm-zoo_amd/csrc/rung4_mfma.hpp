@@ -141,10 +141,13 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
 // wave still reads operands from LDS.
 // BLK = 16: the accumulators are those of the 16x16 instructions, acc[i][j][e] = D(row0 + 16 i + lane % 16,
 // col0 + 16 j + 4 (lane / 16) + e); FM and FN still count 32-row and 32-column blocks.
-template <int TYPES, int FM, int FN, bool RAGGED = false, int BLK = 32, class Acc, int AM, int AN>
+// TRANSPOSED (BLK = 16): the blocks come as acc[j][i], the array of a kernel that ran the transposed problem.
+template <int TYPES, int FM, int FN, bool RAGGED = false, int BLK = 32, bool TRANSPOSED = false, class Acc, int AM, int AN>
 __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g, Acc (&acc)[AM][AN], int row0, int col0,
                                                        int lane, char* region) {
-  static_assert(AM == FM * (32 / BLK) && AN == FN * (32 / BLK), "accumulator blocks of BLK x BLK");
+  static_assert(TRANSPOSED ? (BLK == 16 && AN == FM * 2 && AM == FN * 2)
+                           : (AM == FM * (32 / BLK) && AN == FN * (32 / BLK)), "accumulator blocks of BLK x BLK");
+  constexpr int NJ = TRANSPOSED ? AM : AN;   // 16-column blocks of a row
   using out_t = typename Traits<TYPES>::out_t;
   using acc_t = typename Traits<TYPES>::acc_t;
   constexpr int COLS = FN * 32, PITCH_E = COLS * 4 + 16;
@@ -202,9 +205,9 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
     } else {
       static_for<2>([&](auto h_c) {
         constexpr int H = decltype(h_c)::value;
-        static_for<AN>([&](auto j_c) {
+        static_for<NJ>([&](auto j_c) {
           constexpr int J = decltype(j_c)::value;
-          const Acc& a = acc[2 * I + H][J];
+          const Acc& a = acc[TRANSPOSED ? J : 2 * I + H][TRANSPOSED ? 2 * I + H : J];
           acc_t v[4] = {a[0], a[1], a[2], a[3]};
           __builtin_memcpy(wr + H * 16 * PITCH_E + J * 64, v, 16);
         });
@@ -1003,7 +1006,7 @@ namespace gz {
 // Launcher
 // ---------------------------------------------------------------------------
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N>
-static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipStream_t s) {
+static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipStream_t s, bool transposed = false) {
   const int tiles_m = ceil_div(g.M, BM), tiles_n = ceil_div(g.N, BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(WAVES_M * WAVES_N * 64);
   const size_t lds = 2u * (size_t)(BM + BN) * PITCH;
@@ -1040,6 +1043,23 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
   const dim3 pgrid((unsigned)(ring == 1 ? mfma_persistent_grid((long long)tiles_m * tiles_n, device_compute_units())
                                         : (long long)tiles_m * tiles_n));
   if constexpr (TYPES != GZ_F32F32F32) {
+    // `transposed`: g is the transposed problem of a column-major A with a column-major B (see SWAP in
+    // rung4_mfma_ring16.hpp), a row-major pair for the ring kernel's operands, with the real C and D
+    // (the waves of a tile laid out the other way round as well: the wave count along the real M stays what it is)
+    if (transposed) {
+      if constexpr (TILE_256 && !(is_fp8(TYPES) && WAVES_M * WAVES_N == 8)) {
+        if (ring && shape_class == MFMA_SHAPE_RAGGED_MN)
+          GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, true, false, false, true>), ring_lds, StreamK{});
+        if (ring && !edge)
+          GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, false, false, false, true>), ring_lds, StreamK{});
+      }
+      if constexpr (BM == 128 && BN == 128 && WAVES_M == 2 && WAVES_N == 2 && !is_fp8(TYPES)) {
+        if (ring && !edge)
+          GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, false, false, false, true>), ring_lds, StreamK{});
+      }
+      set_error("mfma rung: no kernel for the transposed problem on this tile");
+      return GZ_ERR_UNSUPPORTED;
+    }
     if constexpr (TILE_256) {
       if (ring && akc && shape_class == MFMA_SHAPE_RAGGED_MN) {
         if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
@@ -1284,7 +1304,8 @@ template <int TYPES> static int launch_strip(const GemmArgs<TYPES>& g, hipStream
   return GZ_OK;
 }
 
-template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& chosen, hipStream_t s, bool adjust = false) {
+template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaCfg& chosen, hipStream_t s, bool adjust = false,
+                                           bool transposed = false) {
   using in_t = typename Traits<TYPES>::in_t;
   MfmaCfg cfg = chosen;
   const int edge = mfma_launch_class(cfg, (int)sizeof(in_t), (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N, g.K,
@@ -1295,11 +1316,11 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
     case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);
     case 3: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 0, s);
     case 4: return launch_cfg<TYPES, 256, 128, 2, 2>(g, edge, 0, s);
-    case 5: case 7: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 1, s);
-    case 6: case 8: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 1, s);
-    case 9: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s);
-    case 10: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s);
-    case 11: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 2, s);
+    case 5: case 7: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 1, s, transposed);
+    case 6: case 8: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 1, s, transposed);
+    case 9: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s, transposed);
+    case 10: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s, transposed);
+    case 11: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 2, s, transposed);
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);
@@ -1342,6 +1363,18 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
   GemmArgs<TYPES> g = args;
   const int num_cus = device_compute_units();
   g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), num_cus);
+  // Column-major A and B: the transposed problem on the ring kernel, where one launch of it covers the problem
+  if (MfmaCfg ct; mfma_transposed_ring(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, num_cus, &ct)) {
+    GemmArgs<TYPES> t = g;
+    t.A = g.B; t.B = g.A;
+    t.M = g.N; t.N = g.M;
+    t.lda = g.ldb; t.ldb = g.lda;
+    t.layoutA = GZ_ROW_MAJOR; t.layoutB = GZ_ROW_MAJOR;
+    const int cls = mfma_launch_class(ct, (int)sizeof(typename Traits<TYPES>::in_t), (int)sizeof(typename Traits<TYPES>::out_t),
+                                      t.M, t.N, t.K, t.layoutA, t.layoutB, t.A, t.B, t.C, t.D, t.lda, t.ldb, t.ldc, t.ldd);
+    // (unaligned operands, or rows of D that are not: the kernels of the problem as given, below)
+    if (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && ct.bm == 256)) return launch_one<TYPES>(t, ct, s, false, true);
+  }
   if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && g.K > 0) {
     StreamKPlan skp;
     const MfmaCfg* forced = variant == 0 ? nullptr : &kMfmaCfgs[variant - 1];

@@ -121,7 +121,13 @@ template <int ES, int ROW_BYTES> __host__ __device__ constexpr int ring16_row_sw
                  : ROW_BYTES >= 256 ? (((r & 7) << 1) ^ ((r >> 4) & 1)) : ((((r >> 1) & 3) << 1) ^ ((r >> 4) & 1));
 }
 
-template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool RAGGED = false, bool STREAMK = false, bool B_KC = true>
+// SWAP: the launch is the transposed problem D^T = B^T A^T of a column-major A with a column-major B.  B^T (N x K,
+// K contiguous) is this kernel's first operand and A^T (K x M, M contiguous) its second, a "row-major B": g.A, g.B,
+// g.M, g.N, g.lda and g.ldb come swapped by the launcher, g.C / g.D / g.ldc / g.ldd are those of the real row-major
+// output.  The MFMAs take their operands in the other order, so that a lane still ends up with four consecutive
+// columns of one row of the real D, and the epilogue walks the accumulator blocks transposed; nothing else changes.
+template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool RAGGED = false, bool STREAMK = false, bool B_KC = true,
+          bool SWAP = false>
 // (second launch bound: waves per SIMD the registers must leave room for - the 128 x 128 tile, whose five buffers are
 // half the LDS, runs two work-groups per compute unit)
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128) ? 2 : (WAVES_M * WAVES_N) / 4)
@@ -141,6 +147,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int HK = 64 / ES;         // K rows of a row-major B per copy group: one K step
   constexpr bool F8 = is_fp8(TYPES);
   static_assert(B_KC || !STREAMK, "stream-K with a column-major B only");
+  static_assert(!SWAP || !B_KC, "the transposed problem of two column-major operands has a row-major second operand");
   static_assert(!(F8 && STREAMK), "stream-K for int8 and the 16-bit types");
   constexpr int A_BYTES = BM / 2 * LINE, B_BYTES = BN / 2 * LINE;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
@@ -363,10 +370,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   // without copies the register allocator no longer kept the accumulators in place across the branches.)
   auto kstep = [&](auto set_c, auto rj_c, auto cp_c, auto cst_c, uint64_t mask, const char* a_src, const char* b_src) {
     constexpr int SET = decltype(set_c)::value, CST = decltype(cst_c)::value;
-#ifndef GZ_X_SPAN
-#define GZ_X_SPAN 1
-#endif
-    constexpr int CPE = NMMA / NCP / GZ_X_SPAN > 0 ? NMMA / NCP / GZ_X_SPAN : 1;                    // MFMAs per copy
+    // MFMAs per copy: over the whole step (bf16 4096^3, us: copies over the whole step 97.7, over its first half
+    // 99.2, all at its start 104.4)
+    constexpr int CPE = NMMA / NCP;
     constexpr int RDE = (NMMA * 3 / 4) / NRD;          // MFMAs per read: the reads end with the third quarter of the step
     static_assert(RDE >= 1, "a step's copies are spread evenly over its MFMAs");
     asm volatile("s_waitcnt lgkmcnt(0)");
@@ -380,13 +386,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     static_for<NMMA>([&](auto q_c) {
       constexpr int Q = decltype(q_c)::value;
       constexpr int I = Q / FN, J = (I & 1) ? FN - 1 - Q % FN : Q % FN;
-      asm_mfma16<TYPES>(acc[I][J], bf[SET][J], af[SET][I]);
+      if constexpr (SWAP) asm_mfma16<TYPES>(acc[I][J], af[SET][I], bf[SET][J]);
+      else asm_mfma16<TYPES>(acc[I][J], bf[SET][J], af[SET][I]);
       if constexpr (Q % RDE == RDE - 1 && Q / RDE < NRD)
         read_one(std::integral_constant<int, SET ^ 1>{}, std::integral_constant<int, Q / RDE>{}, rj_c);
       constexpr int Tc = Q / CPE;
       if constexpr (Q == 0) copy_a_begin(CST);
       if constexpr (Q == CPE * A_PW) copy_b_begin(CST);
-      if constexpr (Q % CPE == CPE / 2 && Tc < NCP) {
+      if constexpr (Q % CPE == CPE / 2) {
         if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, cp_c, a_src, mask);
         else copy_b(std::integral_constant<int, Tc - A_PW>{}, cp_c, b_src, mask);
       }
@@ -434,6 +441,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     constexpr int I = decltype(i_c)::value, J = decltype(j_c)::value;
     if constexpr (B_KC)
       asm_mfma16_f8<TYPES>(acc[I][J], join8(bf[0][J], bf[1][J]), join8(af[0][I], af[1][I]));
+    else if constexpr (SWAP)
+      asm_mfma16_f8<TYPES>(acc[I][J], join8(af[0][I], af[1][I]),
+                           join8(join4(bh[0][J][0], bh[0][J][1]), join4(bh[1][J][0], bh[1][J][1])));
     else
       asm_mfma16_f8<TYPES>(acc[I][J], join8(join4(bh[0][J][0], bh[0][J][1]), join4(bh[1][J][0], bh[1][J][1])),
                            join8(af[0][I], af[1][I]));
@@ -570,8 +580,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   });
 
   // the epilogue passes the accumulators through the end of the operand buffers: 4 and 3 and a little of 2
-  static_assert(NW * epilogue_region_bytes<WN / 32>() <= 3 * STAGE_BYTES, "the epilogue leaves buffers 0 and 1 alone");
-  char* const staging = lds + NST * STAGE_BYTES - (NW - wave) * epilogue_region_bytes<WN / 32>();
+  constexpr int EP_COLS32 = (SWAP ? WM : WN) / 32;   // 32-column blocks of the real D per wave
+  static_assert(NW * epilogue_region_bytes<EP_COLS32>() <= 3 * STAGE_BYTES, "the epilogue leaves buffers 0 and 1 alone");
+  char* const staging = lds + NST * STAGE_BYTES - (NW - wave) * epilogue_region_bytes<EP_COLS32>();
   __syncthreads();   // no wave reads operands any more and no copy is in flight
   if constexpr (PERSISTENT) {
     prefetched = false;
@@ -610,8 +621,15 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     if (!partial || it >= it_end) break;
     __syncthreads();   // the next piece's copies overwrite the buffers the epilogue has just read
   } else {
-    store_accumulators_lds<TYPES, WM / 32, WN / 32, RAGGED, 16>(g, acc, m0 + wm * WM, n0 + wn * WN, lane,
-                                                                staging);
+    if constexpr (SWAP) {
+      GemmArgs<TYPES> gr = g;   // the real output: this kernel's columns are its rows
+      gr.M = g.N;
+      gr.N = g.M;
+      store_accumulators_lds<TYPES, WN / 32, WM / 32, RAGGED, 16, true>(gr, acc, n0 + wn * WN, m0 + wm * WM, lane, staging);
+    } else {
+      store_accumulators_lds<TYPES, WM / 32, WN / 32, RAGGED, 16>(g, acc, m0 + wm * WM, n0 + wn * WN, lane,
+                                                                  staging);
+    }
     if constexpr (!PERSISTENT) break;
     bid += (int)gridDim.x;
     if (bid >= tiles_m * tiles_n) break;

@@ -130,6 +130,38 @@ def test_whole_line_pipeline_every_slab_count(G, types):
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1)), (types, variant, m, n, k)
 
 
+@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.E4M3E4M3F16, O.E5M2E5M2F16))
+def test_whole_line_pipeline_on_the_transposed_problem(G, types):
+    """Column-major A and B: the same kernel runs D^T = B^T A^T (a row-major pair of operands) and writes the
+    row-major D.  Whole tiles on every variant of that kernel, the launcher's own choice, M and N ragged (M in whole
+    16-byte pieces), alpha and beta at work; shapes the kernel cannot take (M = 300) run the kernels of the problem
+    as given.  Bit-exact."""
+    slab = 128 // np.dtype(O.IN_DTYPE[types]).itemsize
+    for variant, slabs, (m, n) in itertools.product((0, 5, 6, 9, 10, 11), (1, 2, 5, 6, 11), [(256, 512), (512, 256), (128, 384)]):
+        k = slab * slabs
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs + 30)
+        print("col/col case", types, variant, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.COL, O.COL, 1, 1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.COL, 1, 1)), (types, variant, m, n, k)
+    for variant, slabs, (m, n) in itertools.product((0, 5, 6), (1, 4, 7), [(528, 300), (240, 257), (16, 511), (300, 528)]):
+        k = slab * slabs
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs + 10)
+        print("ragged col/col case", types, variant, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.COL, O.COL, 2, -1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.COL, 2, -1)), (types, variant, m, n, k)
+    # sub-matrix views: leading dimensions of whole 16-byte pieces stay on this path, odd ones leave it
+    piece_in = 16 // np.dtype(O.IN_DTYPE[types]).itemsize
+    piece_out = 16 // np.dtype(O.OUT_DTYPE[types]).itemsize
+    for variant, (m, n), pads in itertools.product((5, 6, 11), [(512, 256), (528, 300)],
+                                                   [(2 * piece_in, piece_in, piece_out, 2 * piece_out), (piece_in, piece_in, 1, 1),
+                                                    (1, 3, piece_out, piece_out)]):
+        k = 3 * slab
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=variant + 3)
+        print("col/col ld case", types, variant, m, n, k, pads, flush=True)
+        got = G.run_gemm_ld(types, a, b, c, m, n, k, O.COL, O.COL, 1, 1, MFMA, variant, pads)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.COL, 1, 1)), (types, variant, m, n, k, pads)
+
+
 @pytest.mark.parametrize("types", (O.E4M3E4M3F16, O.E5M2E5M2F16))
 def test_whole_line_pipeline_8bit_floats_on_normal_data(G, types):
     """The 16x16x128 kernel (variants 5 and 6) on N(0,1) data, where every bit of the operands matters: a long K
