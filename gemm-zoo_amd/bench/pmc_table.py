@@ -3,8 +3,11 @@
 
     python3 gemm-zoo_amd/bench/pmc_table.py gpurun_out/pmc_a gpurun_out/pmc_b [--skip fill,elementwise]
 
-Every directory is searched for *counter_collection.csv; one line per (kernel, counter): mean over the dispatches
-of that kernel, and the number of dispatches.  Text in, text out: what goes into profiles/ is this output.
+Every directory is searched for *counter_collection.csv; one line per (kernel, counter): mean, minimum and maximum
+over the dispatches of that kernel, and their number.  With --levels the dispatches of a kernel are also grouped by
+value (groups of values within 2 % of each other): a kernel that ran two workloads in one process - with and without
+reading C, a small copy and a large one - shows one line per workload.  Text in, text out: what goes into profiles/
+is this output.
 """
 import argparse
 import collections
@@ -18,6 +21,7 @@ def main() -> int:
     ap.add_argument("dirs", nargs="+")
     ap.add_argument("--skip", default="fill_kernel,elementwise,compare", help="kernel-name substrings to leave out")
     ap.add_argument("--width", type=int, default=96)
+    ap.add_argument("--levels", action="store_true", help="also list the groups of near-equal values per counter")
     args = ap.parse_args()
     skip = [s for s in args.skip.split(",") if s]
     table = collections.OrderedDict()
@@ -33,7 +37,16 @@ def main() -> int:
     for name, counters in table.items():
         print(name[:args.width])
         for c, vals in counters.items():
-            print(f"    {c:40s} {sum(vals) / len(vals):18,.0f}   ({len(vals)} dispatches)")
+            print(f"    {c:40s} {sum(vals) / len(vals):18,.0f}   min {min(vals):,.0f}  max {max(vals):,.0f}  ({len(vals)} dispatches)")
+            if args.levels and max(vals) > 1.02 * min(vals):
+                groups = []
+                for v in sorted(vals):
+                    if groups and v <= 1.02 * groups[-1][0]:
+                        groups[-1].append(v)
+                    else:
+                        groups.append([v])
+                for g in groups:
+                    print(f"        level {sum(g) / len(g):18,.1f}   x {len(g)}")
     return 0
 
 
