@@ -980,15 +980,6 @@ template <int OFF> __device__ __forceinline__ void asm_copy16(uint32_t voff, con
   static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
   asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase), "i"(OFF) : "memory");
 }
-// The same under a lane mask (a scalar register pair): an all-zero mask turns the instruction into a no-op that
-// still takes its place in the sequence and in the vmcnt order.
-template <int OFF> __device__ __forceinline__ void asm_copy16_masked(uint32_t voff, const void* sbase, uint64_t mask) {
-  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed immediate");
-  asm volatile("s_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2\n\ts_mov_b64 exec, -1"
-               :
-               : "v"(voff), "s"(sbase), "i"(OFF), "s"(mask)
-               : "memory");
-}
 typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
 // half a fragment of a row-major B through the transposing LDS reads
 template <int ES, int OFF> __device__ __forceinline__ void asm_ds_read_tr(u32x2_t& dst, uint32_t addr) {

@@ -218,8 +218,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   // row and piece - and the immediate.  The immediate also moves the LDS address (that is what it is for: the copies
   // of a group step through LDS with it, under one M0), so it is taken off the per-lane offset again; COPY_BIAS keeps
   // that difference non-negative and is taken off the scalar base.  (Before: one scalar base per copy, computed in
-  // the loop with four to six scalar instructions, and a lane mask around every copy for the groups past the end of
-  // K - seven to ten instructions per copy between two MFMAs, where a wave that is alone on its SIMD issues one
+  // the loop with four to six scalar instructions, and a compare and a branch around every copy for the groups past
+  // the end of K - seven to ten instructions per copy between two MFMAs, where a wave that is alone on its SIMD issues one
   // instruction every four cycles and an MFMA leaves room for three.)
   constexpr uint32_t COPY_BIAS = 4096;
   const int ci = lane >> 3, cs = lane & 7;
@@ -280,13 +280,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   const uint32_t m0_b = lds_base + A_BYTES + (wave * B_PW) * 1024 + (B_PW / 2) * 1024;
   auto copy_a_begin = [&](int st) { asm_set_m0(m0_a + st * STAGE_BYTES); };
   auto copy_b_begin = [&](int st) { asm_set_m0(m0_b + st * STAGE_BYTES); };
-  auto copy_a = [&](auto t_c, auto p_c, const char* src, uint64_t mask) {
+  auto copy_a = [&](auto t_c, auto p_c, const char* src) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - A_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(voff_a[P][Tn], src, mask);
+    asm_copy16<OFF>(voff_a[P][Tn], src);
   };
-  auto copy_b = [&](auto t_c, auto p_c, const char* src, uint64_t mask) {
+  auto copy_b = [&](auto t_c, auto p_c, const char* src) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - B_PW / 2) * 1024;
-    asm_copy16_masked<OFF>(voff_b[B_KC ? P : 0][Tn], src, mask);
+    asm_copy16<OFF>(voff_b[B_KC ? P : 0][Tn], src);
   };
 
   // ---- fragment addressing: one LDS byte address per (slab position in the ring, K step) ----
@@ -365,10 +365,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   // One K step: NMMA MFMAs on register set SET, rows of blocks walked back and forth so that consecutive
   // instructions share an operand.  Between them the NRD fragment reads of (ring position RJ, K step SET ^ 1) into
   // the other set, and the copies of a group of parity CP into buffer CST from a_src / b_src: the A rows in the first
-  // half, the B rows in the second.  The last two slabs of a run have nothing left to fetch: `mask` (the lanes of a
-  // copy, a scalar register pair) is zero there.  (One body for both cases: with a second instance of the step
-  // without copies the register allocator no longer kept the accumulators in place across the branches.)
-  auto kstep = [&](auto set_c, auto rj_c, auto cp_c, auto cst_c, uint64_t mask, const char* a_src, const char* b_src) {
+  // half, the B rows in the second.  The last two slabs of a run have nothing left to fetch: their copies fetch the
+  // run's last slab once more (a_src / b_src stop advancing there), into buffers that nothing reads any more.  A
+  // copy that is switched off costs more than one that runs: under an all-zero lane mask it still takes its place in
+  // the memory pipeline, and the two writes of exec around it took two of the three issue slots an MFMA leaves -
+  // and a second instance of the step without copies made the register allocator give up the accumulators' places
+  // across the branches (it spilled 950 - 1800 registers).
+  auto kstep = [&](auto set_c, auto rj_c, auto cp_c, auto cst_c, const char* a_src, const char* b_src) {
     constexpr int SET = decltype(set_c)::value, CST = decltype(cst_c)::value;
     // MFMAs per copy: over the whole step (bf16 4096^3, us: copies over the whole step 97.7, over its first half
     // 99.2, all at its start 104.4)
@@ -394,8 +397,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
       if constexpr (Q == 0) copy_a_begin(CST);
       if constexpr (Q == CPE * A_PW) copy_b_begin(CST);
       if constexpr (Q % CPE == CPE / 2) {
-        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, cp_c, a_src, mask);
-        else copy_b(std::integral_constant<int, Tc - A_PW>{}, cp_c, b_src, mask);
+        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, cp_c, a_src);
+        else copy_b(std::integral_constant<int, Tc - A_PW>{}, cp_c, b_src);
       }
     });
   };
@@ -449,7 +452,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
                            join8(af[0][I], af[1][I]));
   };
   // half H of the slab at ring position JR; the copies of a group of parity H into buffer CST as in kstep
-  auto half_f8 = [&](auto h_c, auto jr_c, auto cst_c, uint64_t mask, const char* a_src, const char* b_src) {
+  auto half_f8 = [&](auto h_c, auto jr_c, auto cst_c, const char* a_src, const char* b_src) {
     constexpr int H = decltype(h_c)::value, JR = decltype(jr_c)::value, CST = decltype(cst_c)::value;
     using NEXT = std::integral_constant<int, (JR + 1) % NST>;
     constexpr int CPE = HM / NCP;          // MFMAs per copy
@@ -485,22 +488,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
       if constexpr (Q == 0) copy_a_begin(CST);
       if constexpr (Q == CPE * A_PW) copy_b_begin(CST);
       if constexpr (Q % CPE == CPE / 2) {
-        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, h_c, a_src, mask);
-        else copy_b(std::integral_constant<int, Tc - A_PW>{}, h_c, b_src, mask);
+        if constexpr (Tc < A_PW) copy_a(std::integral_constant<int, Tc>{}, h_c, a_src);
+        else copy_b(std::integral_constant<int, Tc - A_PW>{}, h_c, b_src);
       }
     });
   };
 
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
-  // lane mask of a copy as a scalar register pair: all ones while a < b, zero otherwise
-  auto mask_if_less = [](int a, int b) -> uint64_t {
-    uint64_t m;
-    asm volatile("s_cmp_lt_i32 %1, %2\n\ts_cselect_b64 %0, -1, 0" : "=s"(m) : "s"(a), "s"(b) : "scc");
-    return m;
-  };
-  constexpr uint64_t ALL_LANES = ~0ull;
-
   // ---- prologue: groups 0 .. 3 (slabs 0 and 1; a run of one slab has groups 0 and 1 only) ----
   const char* const a_tile = a_base_of(m0);
   const char* const b_tile = b_base_of(n0);
@@ -509,9 +504,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     const char* const a_src = a_group(a_t, C);
     const char* const b_src = b_group(b_t, C);
     copy_a_begin(C);
-    static_for<A_PW>([&](auto t) { copy_a(t, std::integral_constant<int, C & 1>{}, a_src, ALL_LANES); });
+    static_for<A_PW>([&](auto t) { copy_a(t, std::integral_constant<int, C & 1>{}, a_src); });
     copy_b_begin(C);
-    static_for<B_PW>([&](auto t) { copy_b(t, std::integral_constant<int, C & 1>{}, b_src, ALL_LANES); });
+    static_for<B_PW>([&](auto t) { copy_b(t, std::integral_constant<int, C & 1>{}, b_src); });
   };
   if (!(PERSISTENT && prefetched)) {   // (persistent: groups 0 and 1 went out before the last tile's epilogue)
     issue_group(std::integral_constant<int, 0>{}, a_tile, b_tile);
@@ -537,30 +532,32 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     static_for<NRD>([&](auto r) { read_one(I0{}, r, I0{}); });
   }
 
-  // ---- one slab; JR = j % 5 at compile time.  Slab j fetches slab j + 2 (groups 2j + 4 and 2j + 5) from a_cp / b_cp ----
-  const char* a_cp = a_group(a_tile, 4);
-  const char* b_cp = b_group(b_tile, 4);
+  // ---- one slab; JR = j % 5 at compile time.  Slab j fetches slab j + 2 (groups 2j + 4 and 2j + 5) from a_cp / b_cp,
+  // or, where the run has no such slab, its last slab again ----
   const int nslab = nc / 2;
+  const int first_fetch = min(2, nslab - 1);
+  const char* a_cp = a_group(a_tile, 2 * first_fetch);
+  const char* b_cp = b_group(b_tile, 2 * first_fetch);
   auto slab = [&](auto jr_c, int j) {
     constexpr int JR = decltype(jr_c)::value;
     using NEXT = std::integral_constant<int, (JR + 1) % NST>;
     using ST4 = std::integral_constant<int, (2 * JR + 4) % NST>;
     using ST5 = std::integral_constant<int, (2 * JR + 5) % NST>;
-    const uint64_t mask = mask_if_less(j + 2, nslab);   // slab j + 2 exists
-    if constexpr (F8) half_f8(I0{}, jr_c, ST4{}, mask, a_cp, b_cp);
-    else kstep(I0{}, jr_c, I0{}, ST4{}, mask, a_cp, b_cp);
+    // a row-major B: a group is a K step's rows, the slab's second group lies a step further
+    const char* const b_cp1 = B_KC ? b_cp : b_cp + b_group_step;
+    if constexpr (F8) half_f8(I0{}, jr_c, ST4{}, a_cp, b_cp);
+    else kstep(I0{}, jr_c, I0{}, ST4{}, a_cp, b_cp);
     if (j + 2 < nslab) {  // the copies of group 2j+4 may stay in flight
       if constexpr (NCP == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
-    if constexpr (!B_KC) b_cp += b_group_step;   // a row-major B: a group is a K step's rows
-    if constexpr (F8) half_f8(I1{}, jr_c, ST5{}, mask, a_cp, b_cp);
-    else kstep(I1{}, NEXT{}, I1{}, ST5{}, mask, a_cp, b_cp);
-    a_cp += LINE;
-    if constexpr (B_KC) b_cp += LINE;
-    else b_cp += b_group_step;
+    if constexpr (F8) half_f8(I1{}, jr_c, ST5{}, a_cp, b_cp1);
+    else kstep(I1{}, NEXT{}, I1{}, ST5{}, a_cp, b_cp1);
+    const bool more = j + 3 < nslab;   // the next slab fetches one further
+    a_cp += more ? (size_t)LINE : (size_t)0;
+    b_cp += more ? (B_KC ? (size_t)LINE : 2 * b_group_step) : (size_t)0;
   };
 
   for (int j = 0; j < nslab; j += NST) {
