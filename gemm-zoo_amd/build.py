@@ -100,6 +100,7 @@ def build_benches(verbose=True, jobs=8):
     def one(src: Path):
         exe = out_dir / src.stem
         _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
               f"-I{include}", str(src), "-o", str(exe), f"-L{LIB}", "-lgemmzoo", "-lgemmzoo_hipblaslt",
               "-Wl,-rpath,$ORIGIN/../../lib", "-Wl,-rpath,/opt/rocm/lib"])
         return exe
