@@ -518,13 +518,18 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         return GZ_ERR_UNSUPPORTED;
       }
       if (variant > 1) { set_error("skinny rung has a single variant"); return GZ_ERR_UNSUPPORTED; }
-      SkinnyCfg c = skinny_resolve(m, n, k, num_cus);
+      SkinnyCfg c = skinny_resolve(m, n, k, num_cus, (unsigned long long)ws_limit);
       plan->variant = 1;
       plan->tile_m = c.mb; plan->tile_n = c.cols_per_wg;
       plan->tile_k = c.kind == SKINNY_KIND_TILE ? STREAM_TILE_K_STEP : c.kind == SKINNY_KIND_DTL ? SKINNY_DTL_K_STEP : SKINNY_K_STEP;
       plan->wave_m = c.kind == SKINNY_KIND_TILE ? 32 : c.mb; plan->wave_n = c.cols_per_wave;
       plan->threads = c.threads; plan->split_k = c.split_k; plan->lds_bytes = c.lds_bytes;
       plan->grid = (int64_t)c.grid_n * c.split_k;
+      if (c.kind == SKINNY_KIND_TILE_WIDE) {   // whole rounds of the eight XCDs; a second launch adds the K parts
+        const int per_round = 8 / c.split_k;
+        plan->grid = (int64_t)((c.grid_n + per_round - 1) / per_round) * 8;
+        plan->workspace_bytes = c.workspace_bytes;
+      }
       return GZ_OK;
     }
     default: break;

@@ -23,7 +23,15 @@ constexpr int STREAM_TILE_COLS = 64;
 constexpr int STREAM_TILE_THREADS = 512;
 constexpr int STREAM_TILE_STAGES_1 = 8, STREAM_TILE_STAGES_2 = 4, STREAM_TILE_STAGES_4 = 4;
 
-enum { SKINNY_KIND_REG = 0, SKINNY_KIND_DTL = 1, SKINNY_KIND_TILE = 2 };
+// the same with wide column blocks and a split K (65 ... 128 rows, long K): 64 CB columns per work-group, CB = 2 ... 4,
+// ring depth by CB; a work-group's partial sums are 4 waves x 2 row blocks x CB column blocks x 4 KiB
+constexpr int STREAM_WIDE_MIN_K = 8192;
+constexpr int STREAM_WIDE_MAX_CB = 4;
+constexpr int STREAM_WIDE_STAGES_2 = 4, STREAM_WIDE_STAGES_3 = 3, STREAM_WIDE_STAGES_4 = 3;
+inline int stream_wide_stages(int cb) { return cb == 2 ? STREAM_WIDE_STAGES_2 : cb == 3 ? STREAM_WIDE_STAGES_3 : STREAM_WIDE_STAGES_4; }
+inline long long stream_wide_slot_bytes(int cb) { return 4LL * 2 * cb * 4 * 1024; }
+
+enum { SKINNY_KIND_REG = 0, SKINNY_KIND_DTL = 1, SKINNY_KIND_TILE = 2, SKINNY_KIND_TILE_WIDE = 3 };
 
 struct SkinnyCfg {
   int mb;             // rows of A the kernel instance covers: 16, 32, 64 or 128
@@ -36,6 +44,8 @@ struct SkinnyCfg {
   int k_per_split;
   int kind;           // SKINNY_KIND_*
   int lds_bytes;
+  int cb;             // SKINNY_KIND_TILE_WIDE: 64-column blocks per work-group
+  long long workspace_bytes;   // partial sums of a split K (0: none)
 };
 
 // Decode-shaped problems only: 16-bit float inputs, activations row-major (K
@@ -74,10 +84,59 @@ inline int skinny_balanced_cols(int N, int num_cus, int max_cols) {
   return max_cols;
 }
 
-inline SkinnyCfg skinny_resolve(int M, int N, int K, int num_cus) {
+// Wide column blocks with a split K.  With 64 columns per work-group every compute unit pulls ALL of A from its L2
+// beside its share of B, and at 65 ... 128 rows that, not HBM, sets the time (M = 128, N = 14336, K = 8192: 2 MiB of A
+// and 0.9 MiB of B per compute unit, 60 us where the B stream alone is 42 at the 5.6 TB/s this part streams).  What a work-group takes in of A is
+// rows x its K range, whatever its columns: splitting K in KS parts AND widening the column blocks KS-fold keeps one
+// work-group per compute unit and divides the A traffic by KS.  The partial sums go to a workspace in the order the
+// waves hold them (whole 1 KiB stores) and a second launch adds them in the order of the K parts - a fixed order, no
+// waiting - and applies alpha, beta and the rounding.  Taken for 64 < M <= 128 from K = 8192 on where the column
+// blocks come out at 65 ... 256 columns and the workspace fits.  The first launch then runs at the rate of the B
+// stream (M = 128, N = 14336: 43 us at K = 8192, 75 at 14336); the second costs 10 us: 60.1 -> 56.3 us and
+// 108.5 -> 84.5.
+inline bool skinny_resolve_wide(int M, int N, int K, int num_cus, unsigned long long ws_limit, int* split, int* cols) {
+  if (num_cus <= 0) num_cus = 256;
+  if (M <= 64 || M > SKINNY_MAX_M || K < STREAM_WIDE_MIN_K) return false;
+  // four parts where the column blocks allow it, else two (M = 128, N = 14336, us, two / four parts: K = 8192
+  // 56.0 / 56.3, K = 14336 93.9 / 84.5; at K = 4096 the split loses to the one-launch kernel, 34.2 against 31.6)
+  for (int ks = 4; ks >= 2; ks >>= 1) {
+    if (num_cus % ks || (K / STREAM_TILE_K_STEP) < 8 * ks) continue;
+    const int groups = num_cus / ks;
+    int per = (N + groups - 1) / groups;
+    per = (per + 3) / 4 * 4;
+    if (per <= STREAM_TILE_COLS || per > STREAM_TILE_COLS * STREAM_WIDE_MAX_CB) continue;
+    const int cb = (per + STREAM_TILE_COLS - 1) / STREAM_TILE_COLS;
+    const long long grid_n = (N + per - 1) / per;
+    if ((unsigned long long)(grid_n * ks * stream_wide_slot_bytes(cb)) > ws_limit) continue;
+    *split = ks;
+    *cols = per;
+    return true;
+  }
+  return false;
+}
+
+inline SkinnyCfg skinny_resolve(int M, int N, int K, int num_cus, unsigned long long ws_limit = ~0ULL) {
   SkinnyCfg c;
   c.split_k = 1;
   c.k_per_split = K;
+  c.cb = 1;
+  c.workspace_bytes = 0;
+  int wide_split = 1, wide_cols = 0;
+  if (skinny_resolve_wide(M, N, K, num_cus, ws_limit, &wide_split, &wide_cols)) {
+    c.kind = SKINNY_KIND_TILE_WIDE;
+    c.mb = 128;
+    c.cols_per_wg = wide_cols;
+    c.cb = (wide_cols + STREAM_TILE_COLS - 1) / STREAM_TILE_COLS;
+    c.cols_per_wave = 32 * c.cb;
+    c.waves = STREAM_TILE_THREADS / 64;
+    c.split_k = wide_split;
+    c.k_per_split = K / wide_split;   // (whole 64-element stages are dealt as evenly as they divide)
+    c.lds_bytes = stream_wide_stages(c.cb) * (128 + STREAM_TILE_COLS * c.cb) * STREAM_TILE_ROW_BYTES;
+    c.threads = c.waves * 64;
+    c.grid_n = (N + c.cols_per_wg - 1) / c.cols_per_wg;
+    c.workspace_bytes = (long long)c.grid_n * c.split_k * stream_wide_slot_bytes(c.cb);
+    return c;
+  }
   if (M > SKINNY_REG_MAX_M) {
     c.kind = SKINNY_KIND_TILE;
     c.mb = M <= 32 ? 32 : M <= 64 ? 64 : 128;

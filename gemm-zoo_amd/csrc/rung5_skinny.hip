@@ -21,6 +21,10 @@
 //
 // skinny_reg_kernel (M <= 16, K % 64 == 0 only): the earlier design, B straight into MFMA operand registers.
 //
+// stream_wide_kernel + stream_wide_reduce_kernel (64 < M <= 128, K >= 8192): stream_tile_kernel with column blocks of
+// up to 256 columns and K split in two or four parts, so that a compute unit pulls a part of A instead of all of it;
+// the parts meet in a workspace and a second launch adds them in a fixed order (gz_skinny_cfg.hpp says when).
+//
 // stream_tile_kernel (16 < M <= 128, K % 64 == 0): here the activations no longer fit a wave's registers and every
 // compute unit needs all of them, so they are shared through LDS.  One work-group per compute unit owns up to 64
 // columns.  Four producer waves move stage after stage (64 K elements: A rows and B rows, 128 bytes each, swizzled)
@@ -543,6 +547,197 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_tile_kernel(GemmAr
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The producer / consumer kernel with wide column blocks and a split K, 64 < M <= 128 (see skinny_resolve_wide)
+//   Work-group b serves K part ks = (b % 8) % KS of column group (b / 8) * (8 / KS) + (b % 8) / KS: work-groups go
+//   to the XCDs in turn, so the work-groups of one XCD share a K part of A and its L2 holds that part only.
+//   LDS ring: S stages of [A: 128 rows | B: 64 CB rows] x 128 bytes, swizzled as above.  Producer wave p moves A rows
+//   [32 p, 32 p + 32) and B rows [16 CB p, 16 CB (p + 1)) of every stage.  Consumer wave w: row blocks 2 (w >> 1) and
+//   2 (w >> 1) + 1, the 32-column blocks (w & 1) + 2 c for c < CB, all four k-steps of a stage; the fragments of
+//   k-step t + 1 are requested before the MFMAs of k-step t.
+//   The sums leave as the waves hold them: slot (ks, group) of the workspace, float4 index
+//   (((wave * 2 + r) * CB + c) * 4 + q) * 64 + lane - whole 1 KiB stores; stream_wide_reduce_kernel reads them back in
+//   the same order.
+// ---------------------------------------------------------------------------------------------------------
+template <int TYPES, int CB, int S>
+__global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_wide_kernel(GemmArgs<TYPES> g, int cols_per_wg, int groups, int KS,
+                                                                          float* ws) {
+  constexpr int NCW = 4;
+  extern __shared__ __attribute__((aligned(1024))) char sk_lds[];
+  constexpr int RB = STREAM_TILE_ROW_BYTES, A_ROWS = 128, A_BYTES = A_ROWS * RB, B_ROWS = STREAM_TILE_COLS * CB;
+  constexpr int B_BYTES = B_ROWS * RB, STAGE = A_BYTES + B_BYTES;
+  constexpr int NA = 4, NB = 2 * CB, NCP = NA + NB;   // copies per producer wave and stage
+  constexpr int NRB = 2, NT = 4;
+  static_assert(CB >= 2 && CB <= STREAM_WIDE_MAX_CB, "two to four 64-column blocks");
+  static_assert((S - 2) * NCP < 64, "vmcnt");
+  static_assert(S * STAGE <= 160 * 1024, "LDS");
+  const uint32_t lds_base = (uint32_t)(uintptr_t)sk_lds;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int N = g.N, M = g.M;
+  const int xcd = blockIdx.x % 8;
+  const int ks = xcd % KS, cg = ((int)blockIdx.x / 8) * (8 / KS) + xcd / KS;
+  if (cg >= groups) return;   // the grid is rounded up to whole rounds of the XCDs; before any barrier
+  const int n_base = cg * cols_per_wg;
+  const int n_end = min(n_base + cols_per_wg, N);
+  const size_t rowb = (size_t)g.ldb * 2, rowb_a = (size_t)g.lda * 2;
+  const int nst_all = g.K / STREAM_TILE_K_STEP;
+  const int st_q = nst_all / KS, st_r = nst_all % KS;
+  const int st0 = ks * st_q + min(ks, st_r), nst = st_q + (ks < st_r ? 1 : 0);
+  const int rot = (int)((unsigned)cg % (unsigned)nst);
+
+  if (wave >= NCW) {
+    const int p = wave - NCW;
+    uint32_t voffA[NA], voffB[NB];
+    uint64_t maskB[NB];
+    const int row_in = lane >> 3, pos = lane & 7;
+#pragma unroll
+    for (int j = 0; j < NA; j++) {
+      const int row = (p * NA + j) * 8 + row_in;
+      voffA[j] = (uint32_t)((size_t)min(row, M - 1) * rowb_a) + (pos ^ ((row >> 1) & 7)) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+      const int row = (p * NB + j) * 8 + row_in;
+      const int n = min(n_base + row, N - 1);
+      voffB[j] = (uint32_t)((size_t)(n - n_base) * rowb) + (pos ^ ((row >> 1) & 7)) * 16;
+      maskB[j] = __builtin_amdgcn_ballot_w64(n_base + row < n_end);
+    }
+    const char* sA = reinterpret_cast<const char*>(g.A) + (size_t)st0 * RB;
+    const char* sB = reinterpret_cast<const char*>(g.B) + (size_t)n_base * rowb + (size_t)st0 * RB;
+    int slot = 0;
+    auto issue = [&](int s) {   // a stage past the end: every copy masked off but still counted
+      const bool exists = s < nst;
+      int c = s + rot;
+      if (c >= nst) c -= nst;
+      if (!exists) c = 0;
+      const uint32_t dst = lds_base + (uint32_t)slot * STAGE;
+      slot = slot + 1 == S ? 0 : slot + 1;
+      sk_set_m0(dst + p * (NA * 1024) + 2048);
+      sk_for<NA>([&](auto j_c) {
+        constexpr int J = decltype(j_c)::value;
+        sk_copy16_keep<(J - 2) * 1024>(voffA[J], sA + (size_t)c * RB - (J - 2) * 1024, __builtin_amdgcn_ballot_w64(exists));
+      });
+      sk_set_m0(dst + A_BYTES + p * (NB * 1024) + (NB / 2) * 1024);
+      sk_for<NB>([&](auto j_c) {
+        constexpr int J = decltype(j_c)::value;
+        const uint64_t m = maskB[J] & __builtin_amdgcn_ballot_w64(exists);
+        sk_copy16<(J - NB / 2) * 1024>(voffB[J], sB + (size_t)c * RB - (J - NB / 2) * 1024, m);
+      });
+    };
+    for (int s = 0; s < S - 1; s++) issue(s);
+    for (int i = 0; i < nst; i++) {
+      sk_wait_vm<(S - 2) * NCP>();                 // stage i has landed
+      asm volatile("s_barrier" ::: "memory");     // consumers are done with stage i - 1
+      issue(i + S - 1);
+    }
+    sk_wait_vm<0>();
+    return;
+  }
+
+  // consumers
+  const int r32 = lane & 31, g2 = lane >> 5;
+  const int cbw = wave & 1, rb0 = (wave >> 1) * NRB;
+  uint32_t b_addr[NT], a_addr[NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const int pp = ((2 * t + g2) ^ ((r32 >> 1) & 7)) * 16;
+    a_addr[t] = lds_base + (rb0 * 32 + r32) * RB + pp;
+    b_addr[t] = lds_base + A_BYTES + (cbw * 32 + r32) * RB + pp;
+  }
+  sk_f32x16_t acc[NRB][CB];
+#pragma unroll
+  for (int r = 0; r < NRB; r++)
+#pragma unroll
+    for (int c = 0; c < CB; c++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[r][c][e] = 0.f;
+
+  uint32_t so = 0;
+  for (int i = 0; i < nst; i++) {
+    asm volatile("s_barrier" ::: "memory");
+    sk_u32x4_t bf[2][CB], af[2][NRB];
+    auto request = [&](auto t_c) {
+      constexpr int TT = decltype(t_c)::value;
+      sk_for<NRB>([&](auto r_c) {
+        constexpr int R = decltype(r_c)::value;
+        sk_ds_read16<R * 32 * RB>(af[TT & 1][R], a_addr[TT] + so);
+      });
+      sk_for<CB>([&](auto c_c) {
+        constexpr int C = decltype(c_c)::value;
+        sk_ds_read16<C * 64 * RB>(bf[TT & 1][C], b_addr[TT] + so);
+      });
+    };
+    request(std::integral_constant<int, 0>{});
+    sk_for<NT>([&](auto t_c) {
+      constexpr int TT = decltype(t_c)::value;
+      if constexpr (TT + 1 < NT) {
+        request(std::integral_constant<int, TT + 1>{});
+        sk_wait_lgkm<NRB + CB>();
+      } else {
+        sk_wait_lgkm0();
+      }
+#pragma unroll
+      for (int r = 0; r < NRB; r++) sk_touch(af[TT & 1][r]);
+#pragma unroll
+      for (int c = 0; c < CB; c++) sk_touch(bf[TT & 1][c]);
+#pragma unroll
+      for (int r = 0; r < NRB; r++)
+#pragma unroll
+        for (int c = 0; c < CB; c++) acc[r][c] = mfma32x16<TYPES>(bf[TT & 1][c], af[TT & 1][r], acc[r][c]);
+    });
+    so = so + STAGE == S * STAGE ? 0 : so + STAGE;
+  }
+
+  sk_f32x4_t* out = reinterpret_cast<sk_f32x4_t*>(ws) +
+                    ((size_t)ks * groups + cg) * (size_t)(NCW * NRB * CB * 4 * 64) + (size_t)wave * (NRB * CB * 4 * 64) + lane;
+#pragma unroll
+  for (int r = 0; r < NRB; r++)
+#pragma unroll
+    for (int c = 0; c < CB; c++)
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        out[((r * CB + c) * 4 + q) * 64] = sk_f32x4_t{acc[r][c][4 * q], acc[r][c][4 * q + 1], acc[r][c][4 * q + 2], acc[r][c][4 * q + 3]};
+}
+
+// Second launch of the split: one lane per four consecutive outputs, in the order the first launch stored them (so
+// that the reads are whole lines); the K parts are added in their order, then alpha, beta and the rounding.
+template <int TYPES>
+__global__ void __launch_bounds__(256) stream_wide_reduce_kernel(GemmArgs<TYPES> g, int cols_per_wg, int groups, int KS, int CB,
+                                                                 const float* ws) {
+  using out_t = typename Traits<TYPES>::out_t;
+  const int per_slot = 4 * 2 * CB * 4 * 64;   // float4 per slot
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int cg = (int)(gid / per_slot), idx = (int)(gid % per_slot);
+  if (cg >= groups) return;
+  const int lane = idx % 64, q = (idx / 64) % 4, c = (idx / 256) % CB, r = (idx / (256 * CB)) % 2, wave = idx / (256 * CB * 2);
+  const int m = ((wave >> 1) * 2 + r) * 32 + (lane & 31);
+  const int n = cg * cols_per_wg + ((wave & 1) + 2 * c) * 32 + q * 8 + (lane >> 5) * 4;
+  const int n_end = min((cg + 1) * cols_per_wg, g.N);
+  if (m >= g.M || n >= n_end) return;
+  const sk_f32x4_t* in = reinterpret_cast<const sk_f32x4_t*>(ws) + (size_t)cg * per_slot + idx;
+  sk_f32x4_t sum = in[0];
+  for (int ks = 1; ks < KS; ks++) {
+    const sk_f32x4_t v = in[(size_t)ks * groups * per_slot];
+#pragma unroll
+    for (int e = 0; e < 4; e++) sum[e] += v[e];
+  }
+  const size_t o = (size_t)m * (size_t)g.ldd + n, oc = (size_t)m * (size_t)g.ldc + n;
+  const bool vec_ok = (g.ldd % 4 == 0) && (g.beta == 0 || g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
+                      (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
+  if (vec_ok && n + 3 < n_end) {
+    out_t cv[4] = {0, 0, 0, 0}, dv[4];
+    if (g.beta != 0) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
+#pragma unroll
+    for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, &cv[e]);
+    __builtin_memcpy(g.D + o, dv, sizeof(dv));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, g.C + oc + e);
+  }
+}
+
 template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hipStream_t s) {
   if constexpr (TYPES == GZ_S8S8S32 || TYPES == GZ_F32F32F32 || is_fp8(TYPES) || is_acc16(TYPES)) {
     (void)g; (void)variant; (void)s;
@@ -563,9 +758,26 @@ template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hi
                 "(lda=%lld ldb=%lld)", (long long)g.lda, (long long)g.ldb);
       return GZ_ERR_UNSUPPORTED;
     }
-    const SkinnyCfg c = skinny_resolve(g.M, g.N, g.K, device_compute_units());
+    const SkinnyCfg c = skinny_resolve(g.M, g.N, g.K, device_compute_units(), (unsigned long long)workspace_limit());
     const dim3 grid((unsigned)c.grid_n), block((unsigned)c.threads);
-    if (c.kind == SKINNY_KIND_TILE) {
+    if (c.kind == SKINNY_KIND_TILE_WIDE) {
+      void* ws = nullptr;
+      const int st = workspace_acquire((size_t)c.workspace_bytes, s, &ws);
+      if (st != GZ_OK) return st;
+      const int per_round = 8 / c.split_k;   // column groups per round of the eight XCDs
+      const dim3 wgrid((unsigned)((c.grid_n + per_round - 1) / per_round * 8));
+      auto k2 = stream_wide_kernel<TYPES, 2, STREAM_WIDE_STAGES_2>;
+      auto k3 = stream_wide_kernel<TYPES, 3, STREAM_WIDE_STAGES_3>;
+      auto k4 = stream_wide_kernel<TYPES, 4, STREAM_WIDE_STAGES_4>;
+      auto kern = c.cb == 2 ? k2 : c.cb == 3 ? k3 : k4;
+      GZ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     c.lds_bytes));
+      hipLaunchKernelGGL(kern, wgrid, block, c.lds_bytes, s, g, c.cols_per_wg, c.grid_n, c.split_k, static_cast<float*>(ws));
+      GZ_HIP_TRY(hipGetLastError());
+      const long long lanes = (long long)c.grid_n * (stream_wide_slot_bytes(c.cb) / 16);
+      hipLaunchKernelGGL((stream_wide_reduce_kernel<TYPES>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, s, g,
+                         c.cols_per_wg, c.grid_n, c.split_k, c.cb, static_cast<const float*>(ws));
+    } else if (c.kind == SKINNY_KIND_TILE) {
       auto k1 = stream_tile_kernel<TYPES, 1, STREAM_TILE_STAGES_1>;
       auto k2 = stream_tile_kernel<TYPES, 2, STREAM_TILE_STAGES_2>;
       auto k4 = stream_tile_kernel<TYPES, 4, STREAM_TILE_STAGES_4>;

@@ -230,3 +230,21 @@ def test_leading_dimension_arguments(capi):
     # 65536 x 65536 x 32768 holds 2^31 and 2^32 elements per matrix: planned like any other problem
     p = capi.plan(capi.S8S8S32, 65536, 65536, 32768, 0, 1)
     assert p.rung == capi.RUNG_MFMA and (p.tile_m, p.tile_n) == (256, 256)
+
+
+def test_plan_skinny_split_k(capi):
+    """The weight-streaming rung splits K for 65 ... 128 rows from K = 8192 on, with column blocks of up to 256
+    columns, and says so in the plan (gz_skinny_cfg.hpp: skinny_resolve_wide)."""
+    p = capi.plan(capi.BF16BF16F32, 128, 14336, 8192, capi.ROW_MAJOR, capi.COL_MAJOR, capi.RUNG_SKINNY, 0, 256, 160 * 1024)
+    assert (p.split_k, p.tile_m, p.tile_n, p.threads) == (4, 128, 224, 512)
+    assert p.grid == 256 and p.workspace_bytes == 256 * 4 * 2 * 4 * 4 * 1024 and p.lds_bytes == 3 * (128 + 256) * 128
+    p = capi.plan(capi.BF16BF16F32, 100, 28672, 8192, capi.ROW_MAJOR, capi.COL_MAJOR, capi.RUNG_SKINNY, 0, 256, 160 * 1024)
+    assert (p.split_k, p.tile_n) == (2, 224)
+    p = capi.plan(capi.BF16BF16F32, 128, 8192, 16384, capi.ROW_MAJOR, capi.COL_MAJOR, capi.RUNG_SKINNY, 0, 256, 160 * 1024)
+    assert (p.split_k, p.tile_n, p.lds_bytes) == (4, 128, 4 * (128 + 128) * 128)
+    for m, n, k in [(64, 14336, 8192), (128, 14336, 4096), (128, 4096, 8192), (128, 65536, 8192)]:
+        p = capi.plan(capi.BF16BF16F32, m, n, k, capi.ROW_MAJOR, capi.COL_MAJOR, capi.RUNG_SKINNY, 0, 256, 160 * 1024)
+        assert p.split_k == 1 and p.workspace_bytes == 0, (m, n, k)
+    # the entry point that allocates nothing: the split only while its partial sums fit the static buffer
+    p = capi.plan_static_scratch(capi.BF16BF16F32, 128, 14336, 8192, capi.ROW_MAJOR, capi.COL_MAJOR, capi.RUNG_SKINNY, 0, 256, 160 * 1024)
+    assert p.split_k == 4 and p.workspace_bytes <= capi.STATIC_SCRATCH_BYTES

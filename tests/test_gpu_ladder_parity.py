@@ -213,6 +213,37 @@ def test_skinny_rung(G, types):
         G.assert_within(types, got, truth, f"skinny {types} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("types", SKINNY_TYPES)
+def test_skinny_rung_long_k_wide_column_blocks(G, types):
+    """65 ... 128 rows with K >= 8192: column blocks of 128 ... 256 columns, K split in two or four parts, partial sums
+    through the workspace and a second launch that adds them in order.  Column counts that fill, nearly fill and
+    barely touch the blocks, K parts of unequal length, alpha / beta, sub-matrix views; M = 64 and K = 4096 beside
+    them stay on the one-launch kernel.  Integer-valued data: every partial sum is exact, so bit-exact."""
+    cases = [(128, 14336, 8192), (100, 8192 + 4, 8192), (65, 12000, 8192 + 64), (128, 4100, 14336), (127, 28672, 8192),
+             (64, 14336, 8192), (128, 14336, 4096)]
+    for (m, n, k), (al, be) in itertools.product(cases, [(1, 0), (0.5, 2)]):
+        plan = G.capi.plan(types, m, n, k, O.ROW, O.COL, SKINNY)
+        assert (plan.split_k > 1) == (m > 64 and k >= 8192), (m, n, k, plan.split_k)
+        assert (plan.workspace_bytes > 0) == (plan.split_k > 1)
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=m + 1)
+        print("case", types, m, n, k, al, be, plan.split_k, plan.tile_n, flush=True)
+        ref = O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, al, be)
+        for rung in (SKINNY, -1):
+            got = G.run_gemm(types, a, b, c, m, n, k, O.ROW, O.COL, al, be, rung)
+            assert np.array_equal(got, ref), (types, m, n, k, al, be, rung)
+    m, n, k = 96, 9000, 8192
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=3)
+    ref = O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1)
+    for pads in [(8, 16, 4, 8), (16, 8, 1, 3)]:
+        assert np.array_equal(G.run_gemm_ld(types, a, b, c, m, n, k, O.ROW, O.COL, 1, 1, SKINNY, 0, pads), ref), pads
+    # N(0,1) activations against weights of N(0, 0.02): within the type's tolerance of the fp64 truth
+    m, n, k = 128, 14336, 8192
+    a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_NORMAL, seed=9, scale_b=0.02)
+    got = G.run_gemm(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0, -1)
+    truth, _ = O.gemm_f64(types, a, b, None, m, n, k, O.ROW, O.COL, 1, 0)
+    G.assert_within(types, got, truth, f"skinny long K {types}")
+
+
 def test_skinny_rung_refuses_what_it_cannot_do(G):
     a = torch.zeros(129 * 64, dtype=torch.int16, device="cuda")
     for kw in (dict(m=129), dict(lb=O.ROW), dict(k=96), dict(types=O.S8S8S32), dict(types=O.F32F32F32),

@@ -21,14 +21,14 @@ def G():
     return gpu_util
 
 
-def run(G, entry, types, a, b, c, m, n, k, alpha, beta, variant):
+def run(G, entry, types, a, b, c, m, n, k, alpha, beta, variant, rung=MFMA):
     """D of one call through `entry` (capi.gemm or capi.gemm_static_scratch), with guard words around it."""
     da, db, dc = G.up(a), G.up(b), G.up(c)
     sentinel = 0x5A5A if O.OUT_DTYPE[types] == np.uint16 else 0x5A5A5A5A
     guard = 64
     full = torch.full((m * n + 2 * guard,), sentinel, dtype=G.out_torch_dtype(types), device=G.dev())
     dd = full[guard:guard + m * n]
-    entry(types, da, db, dc, dd, m, n, k, O.ROW, O.COL, alpha, beta, MFMA, variant,
+    entry(types, da, db, dc, dd, m, n, k, O.ROW, O.COL, alpha, beta, rung, variant,
           torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     host = full.cpu()
@@ -59,6 +59,23 @@ def test_two_calls_in_a_row_match_gz_gemm(G, types, kind):
         else:                    # within the bundle's tolerance of the fp64 truth
             truth, _ = O.gemm_f64(types, a, b, c, m, n, k, O.ROW, O.COL, 2.0, -1.0)
             G.assert_within(types, got, truth, f"static scratch {types} {m}x{n}x{k}")
+
+
+def test_split_k_of_the_streaming_rung_uses_the_same_buffer(G):
+    """The weight-streaming rung's split K (65 ... 128 rows, K >= 8192) leaves its partial sums in the same static
+    buffer: two calls in a row, the second smaller, against gz_gemm bit for bit and against the oracle."""
+    capi = G.capi
+    types = O.BF16BF16F32
+    outs = []
+    for (m, n, k) in [(128, 14336, 8192), (96, 8200, 8192)]:
+        p = capi.plan_static_scratch(types, m, n, k, O.ROW, O.COL, 5, 0)
+        assert p.split_k > 1 and 0 < p.workspace_bytes <= capi.STATIC_SCRATCH_BYTES, p.as_dict()
+        a, b, c = O.make_inputs(types, m, n, k, kind=O.FILL_SMALL_INT, seed=m)
+        print("static scratch, streaming rung", m, n, k, flush=True)
+        outs.append((run(G, capi.gemm_static_scratch, types, a, b, c, m, n, k, 2, -1, 0, rung=5), (a, b, c, m, n, k)))
+    for got, (a, b, c, m, n, k) in outs:
+        assert np.array_equal(got, run(G, capi.gemm, types, a, b, c, m, n, k, 2, -1, 0, rung=5)), (m, n, k)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.COL, 2, -1)), (m, n, k)
 
 
 def test_more_than_the_buffer_holds_is_refused(G):
