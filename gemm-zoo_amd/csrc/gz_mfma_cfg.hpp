@@ -396,6 +396,11 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
     // a smaller tile was preferred for the whole problem (few tiles): stream-K still competes, on the 256 x 256 tile
     cfg = kMfmaCfgs[in_size == 2 ? MFMA_CFG_RING_W8 : MFMA_CFG_RING_W4];
   }
+  // Below one round of tiles every work-group is a piece whose sums leave as fp32 whatever the output type, so the
+  // eight waves' faster 16-bit epilogue does not apply and four waves' cheaper main loop does (bf16 -> f32, us, four /
+  // eight waves: 1024^2 x 8192 43.6 / 46.1, 1280^2 x 8192 56.4 / 61.0, 2048^2 x 8192 72.6 / 77.5, x 16384
+  // 113.8 / 124.2).
+  if (!forced && (long long)((M + 255) / 256) * ((N + 255) / 256) < num_cus) cfg = kMfmaCfgs[MFMA_CFG_RING_W4];
   if (mfma_shape_class(cfg, in_size, M, N, K, layoutA, layoutB) == MFMA_SHAPE_GENERAL) return false;
   const int nslab = K / (MFMA_SLAB_BYTES / in_size);
   const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
@@ -443,7 +448,12 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
   // 149 / 158; 2048^2 (64) - , - , 76.0 / 79.7, 126 / 167; 2560^2 (100) at 8192 147 / 112 (256 x 128 tiles);
   // int8 (slabs of 128 K) 768^2 at K = 4096 31.3 / 18.2, 8192 24.6 / 31.4; 1536^2 at 8192 49.1 / 34.1,
   // 16384 68.3 / 62.5.  In slabs: at least 48 and at least four per tile of the grid.
-  if (full == 0 && nslab < (4 * R > 48 ? 4 * R : 48)) return false;
+  // Where the runs are whole fractions of a tile - every work-group one piece, none that ends one tile and begins the
+  // next with a second 256 KiB store - two slabs per tile of the grid are enough (2048^2 x 8192: 64 tiles in quarters,
+  // 72.6 us against 82.6 on 128 x 128 tiles; 1792^2 x 8192, 49 tiles in runs of 24.5 slabs: 85.5 against 79.7).
+  const bool whole_fractions = out->rem == 0 && nslab % out->q == 0;
+  const int per_tile = whole_fractions ? 2 : 4;
+  if (full == 0 && nslab < (per_tile * R > 48 ? per_tile * R : 48)) return false;
   // past whole rounds only where few tiles remain: between an eighth and most of a round the estimates of the
   // alternatives are not sharp enough to tell (4608^3: 180 us with the rows cut in two launches, 188 here)
   // (two whole rounds and a quarter: 6144^2 x 4096, 64 of 576 tiles remain, 248 us against 268 in one plain launch)

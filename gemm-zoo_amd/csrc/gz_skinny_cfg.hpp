@@ -92,13 +92,13 @@ inline int skinny_balanced_cols(int N, int num_cus, int max_cols) {
 // waves hold them (whole 1 KiB stores) and a second launch adds them in the order of the K parts - a fixed order, no
 // waiting - and applies alpha, beta and the rounding.  Taken for 64 < M <= 128 from K = 8192 on where the column
 // blocks come out at 65 ... 256 columns and the workspace fits.  The first launch then runs at the rate of the B
-// stream (M = 128, N = 14336: 43 us at K = 8192, 75 at 14336); the second costs 10 us: 60.1 -> 56.3 us and
-// 108.5 -> 84.5.
+// stream (M = 128, N = 14336: 43 us at K = 8192, 75 at 14336); the second costs 8 us: 60.1 -> 53.9 us and
+// 108.5 -> 83.1.
 inline bool skinny_resolve_wide(int M, int N, int K, int num_cus, unsigned long long ws_limit, int* split, int* cols) {
   if (num_cus <= 0) num_cus = 256;
   if (M <= 64 || M > SKINNY_MAX_M || K < STREAM_WIDE_MIN_K) return false;
   // four parts where the column blocks allow it, else two (M = 128, N = 14336, us, two / four parts: K = 8192
-  // 56.0 / 56.3, K = 14336 93.9 / 84.5; at K = 4096 the split loses to the one-launch kernel, 34.2 against 31.6)
+  // 56.0 / 56.3, K = 14336 93.9 / 84.5, before the second launch wrote whole rows; at K = 4096 the split loses to the one-launch kernel, 34.2 against 31.6)
   for (int ks = 4; ks >= 2; ks >>= 1) {
     if (num_cus % ks || (K / STREAM_TILE_K_STEP) < 8 * ks) continue;
     const int groups = num_cus / ks;

@@ -700,28 +700,39 @@ __global__ void __launch_bounds__(STREAM_TILE_THREADS) stream_wide_kernel(GemmAr
         out[((r * CB + c) * 4 + q) * 64] = sk_f32x4_t{acc[r][c][4 * q], acc[r][c][4 * q + 1], acc[r][c][4 * q + 2], acc[r][c][4 * q + 3]};
 }
 
-// Second launch of the split: one lane per four consecutive outputs, in the order the first launch stored them (so
-// that the reads are whole lines); the K parts are added in their order, then alpha, beta and the rounding.
+// Second launch of the split: a work-group per 32 x 32 block of the output.  Its 256 lanes read the block's sums in
+// the order the first launch stored them (whole lines), add the K parts in their order, turn the block through LDS
+// and write it row by row - eight lanes per row, 128 contiguous bytes of an fp32 D - with alpha, beta and the rounding.
+// (One lane per four outputs in storage order, each lane writing its own 16 bytes, took 10 us at M = 128, N = 14336:
+// a wave's store then touched 32 rows.)
 template <int TYPES>
 __global__ void __launch_bounds__(256) stream_wide_reduce_kernel(GemmArgs<TYPES> g, int cols_per_wg, int groups, int KS, int CB,
                                                                  const float* ws) {
   using out_t = typename Traits<TYPES>::out_t;
+  __shared__ float tile[32][36];
   const int per_slot = 4 * 2 * CB * 4 * 64;   // float4 per slot
-  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-  const int cg = (int)(gid / per_slot), idx = (int)(gid % per_slot);
-  if (cg >= groups) return;
-  const int lane = idx % 64, q = (idx / 64) % 4, c = (idx / 256) % CB, r = (idx / (256 * CB)) % 2, wave = idx / (256 * CB * 2);
-  const int m = ((wave >> 1) * 2 + r) * 32 + (lane & 31);
-  const int n = cg * cols_per_wg + ((wave & 1) + 2 * c) * 32 + q * 8 + (lane >> 5) * 4;
-  const int n_end = min((cg + 1) * cols_per_wg, g.N);
-  if (m >= g.M || n >= n_end) return;
-  const sk_f32x4_t* in = reinterpret_cast<const sk_f32x4_t*>(ws) + (size_t)cg * per_slot + idx;
+  const int blocks_per_slot = 4 * 2 * CB;
+  const int cg = (int)blockIdx.x / blocks_per_slot, blk = (int)blockIdx.x % blocks_per_slot;
+  const int c = blk % CB, r = (blk / CB) % 2, wave = blk / (2 * CB);
+  const int tid = threadIdx.x, lane = tid % 64, q = tid / 64;
+  const sk_f32x4_t* in = reinterpret_cast<const sk_f32x4_t*>(ws) + (size_t)cg * per_slot + (size_t)blk * 256 + tid;
   sk_f32x4_t sum = in[0];
   for (int ks = 1; ks < KS; ks++) {
     const sk_f32x4_t v = in[(size_t)ks * groups * per_slot];
 #pragma unroll
     for (int e = 0; e < 4; e++) sum[e] += v[e];
   }
+#pragma unroll
+  for (int e = 0; e < 4; e++) tile[lane & 31][q * 8 + (lane >> 5) * 4 + e] = sum[e];
+  __syncthreads();
+  const int row = tid / 8, j = tid % 8;
+  const int m = ((wave >> 1) * 2 + r) * 32 + row;
+  const int n = cg * cols_per_wg + ((wave & 1) + 2 * c) * 32 + 4 * j;
+  const int n_end = min((cg + 1) * cols_per_wg, g.N);
+  if (m >= g.M || n >= n_end) return;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) v[e] = tile[row][4 * j + e];
   const size_t o = (size_t)m * (size_t)g.ldd + n, oc = (size_t)m * (size_t)g.ldc + n;
   const bool vec_ok = (g.ldd % 4 == 0) && (g.beta == 0 || g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(g.D) & 15u) == 0) &&
                       (g.beta == 0 || (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0);
@@ -729,12 +740,12 @@ __global__ void __launch_bounds__(256) stream_wide_reduce_kernel(GemmArgs<TYPES>
     out_t cv[4] = {0, 0, 0, 0}, dv[4];
     if (g.beta != 0) __builtin_memcpy(cv, g.C + oc, sizeof(cv));
 #pragma unroll
-    for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, &cv[e]);
+    for (int e = 0; e < 4; e++) dv[e] = epilogue<TYPES>(v[e], g.alpha, g.beta, &cv[e]);
     __builtin_memcpy(g.D + o, dv, sizeof(dv));
   } else {
 #pragma unroll
     for (int e = 0; e < 4; e++)
-      if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(sum[e], g.alpha, g.beta, g.C + oc + e);
+      if (n + e < n_end) g.D[o + e] = epilogue<TYPES>(v[e], g.alpha, g.beta, g.C + oc + e);
   }
 }
 
@@ -774,8 +785,7 @@ template <int TYPES> int launch_skinny(const GemmArgs<TYPES>& g, int variant, hi
                                      c.lds_bytes));
       hipLaunchKernelGGL(kern, wgrid, block, c.lds_bytes, s, g, c.cols_per_wg, c.grid_n, c.split_k, static_cast<float*>(ws));
       GZ_HIP_TRY(hipGetLastError());
-      const long long lanes = (long long)c.grid_n * (stream_wide_slot_bytes(c.cb) / 16);
-      hipLaunchKernelGGL((stream_wide_reduce_kernel<TYPES>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, s, g,
+      hipLaunchKernelGGL((stream_wide_reduce_kernel<TYPES>), dim3((unsigned)(c.grid_n * 4 * 2 * c.cb)), dim3(256), 0, s, g,
                          c.cols_per_wg, c.grid_n, c.split_k, c.cb, static_cast<const float*>(ws));
     } else if (c.kind == SKINNY_KIND_TILE) {
       auto k1 = stream_tile_kernel<TYPES, 1, STREAM_TILE_STAGES_1>;
