@@ -253,6 +253,10 @@ def main() -> int:
         rr = timed(capi.BF16BF16F32, M, N, K, capi.ROW_MAJOR, capi.ROW_MAJOR, args.steps, args.warmup)
         extras["bf16_4096_row_row"] = {"tflops": round(flops / (rr["kernel_ms_mean"] * 1e-3) / 1e12, 2),
                                        "kernel_ms_mean": round(rr["kernel_ms_mean"], 5)}
+        # column-major A with column-major B: the same kernel on the transposed problem
+        rc = timed(capi.BF16BF16F32, M, N, K, capi.COL_MAJOR, capi.COL_MAJOR, args.steps, args.warmup)
+        extras["bf16_4096_col_col"] = {"tflops": round(flops / (rc["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                                       "kernel_ms_mean": round(rc["kernel_ms_mean"], 5)}
         # next row of the scope: fp8 e4m3 x e4m3 -> fp16 (the reference times cuBLASLt on it,
         # nvidia/bench/bench_cublaslt_e4m3.cu:6-21), this library's own kernel on the reference drivers' layout
         # (row-major A and B); inputs N(0, 0.25) so that the fp16 outputs of K = 8192 stay far from overflow
@@ -302,6 +306,11 @@ def main() -> int:
             sk[f"M={m}"] = {"gb_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
                             "kernel_us_mean": round(rs["kernel_ms_mean"] * 1e3, 2)}
         extras["skinny_bf16_N14336_K4096"] = sk
+        # a long K at 128 rows: the K split with wide column blocks (two launches, partial sums in the workspace)
+        rs = timed(capi.BF16BF16BF16, 128, 14336, 14336, capi.ROW_MAJOR, capi.COL_MAJOR, 30, 60, scale_b=0.02)
+        gbs = rs["problem_bytes"] / (rs["kernel_ms_mean"] * 1e-3) / 1e9
+        extras["skinny_bf16_M128_N14336_K14336"] = {"gb_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                                                    "kernel_us_mean": round(rs["kernel_ms_mean"] * 1e3, 2)}
         out["extras"] = extras
 
     # ---------------- CPU restatement of the reference GEMM on this box's host cores ----------------

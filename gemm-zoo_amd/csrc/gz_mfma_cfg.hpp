@@ -58,7 +58,8 @@ inline int mfma_shape_class(const MfmaCfg& c, int in_size, int M, int N, int K, 
   // the direct-to-LDS kernels address a tile's rows with 32-bit byte offsets from the tile's first row
   if ((long long)K * in_size * 256 >= (1LL << 32) || (long long)N * in_size * 256 >= (1LL << 32)) return MFMA_SHAPE_GENERAL;
   if (M % c.bm == 0 && N % c.bn == 0) return MFMA_SHAPE_WHOLE;
-  if (layoutA != GZ_ROW_MAJOR) return MFMA_SHAPE_GENERAL;
+  // ragged M / N: lines that are not K-contiguous are clamped by whole 16-byte pieces
+  if (layoutA != GZ_ROW_MAJOR && (layoutB != GZ_ROW_MAJOR || M % epv)) return MFMA_SHAPE_GENERAL;
   if (layoutB == GZ_ROW_MAJOR && N % epv) return MFMA_SHAPE_GENERAL;
   return MFMA_SHAPE_RAGGED_MN;
 }
@@ -113,8 +114,12 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   const int in_size = mfma_in_size(types);
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
   // candidates: 256x256 (on the ring kernel where the types and the layout of A allow it), 256x128, 128x128
-  const bool ring_ok = a_rows && types != GZ_F32F32F32;
-  const bool ring128_ok = ring_ok && types != GZ_E4M3E4M3F16 && types != GZ_E5M2E5M2F16;
+  // (a column-major A beside a row-major B goes through the transposing reads like B, not for the 8-bit floats; beside
+  // a column-major B the launcher runs the transposed problem where it can, see mfma_transposed_ring)
+  const bool f8_types = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
+  const bool a_direct = a_rows || (!b_cols && !f8_types);
+  const bool ring_ok = a_direct && types != GZ_F32F32F32;
+  const bool ring128_ok = ring_ok && !f8_types;
   const int cand[3] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,
                        ring128_ok ? MFMA_CFG_RING_128 : MFMA_CFG_128};
   double best = 0;
@@ -125,7 +130,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const long long rounds = (tiles + num_cus - 1) / num_cus;
     // whole tiles: every candidate has a direct-to-LDS kernel; ragged M or N: the 256x256 ones only
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
-    const bool direct = a_rows && types != GZ_F32F32F32 &&
+    const bool direct = a_direct && types != GZ_F32F32F32 &&
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     // (128 x 128 beyond four rounds: each further round costs a little more, 6144^2 x 6144 = 9 rounds measured
     // 478 us against 457 for three rounds of 256 x 256)
@@ -249,12 +254,13 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
 // kernel (ragged K, unaligned operands) wants eight waves for 8-bit integers and 16-bit floats with a row-major A
 // (4096 x 4096 x 4000, us, four / eight waves: int8 96 / 82 and 103 / 84 with a row-major B, bf16 161 / 133 and
 // 180 / 149) and four for the 8-bit floats, whose eight-wave instance does not fit its registers (105 / 206).
-inline void mfma_adjust_general(int types, int cls, int layoutA, MfmaCfg* c) {
+inline void mfma_adjust_general(int types, int cls, int layoutA, int layoutB, MfmaCfg* c) {
   // (whole tiles of a column-major A are in the "whole" class and still run on that kernel; they gain as well:
   // 4096^3, int8 84 / 77, bf16 135 / 124 and 144 / 128 with a row-major B)
-  const bool staged = cls == MFMA_SHAPE_GENERAL || layoutA != GZ_ROW_MAJOR;
-  if (!staged || c->bm != 256 || c->bn != 256) return;
   const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
+  const bool a_staged = layoutA != GZ_ROW_MAJOR && (layoutB != GZ_ROW_MAJOR || f8 || types == GZ_F32F32F32);
+  const bool staged = cls == MFMA_SHAPE_GENERAL || a_staged;
+  if (!staged || c->bm != 256 || c->bn != 256) return;
   if (f8) *c = kMfmaCfgs[MFMA_CFG_256_W4];
   else if (types != GZ_F32F32F32) *c = kMfmaCfgs[MFMA_CFG_256_W8];
   else *c = kMfmaCfgs[MFMA_CFG_256_W4];
@@ -519,7 +525,8 @@ inline int mfma_launch_class(const MfmaCfg& c, int in_size, int out_size, int M,
   int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
   if (cls == MFMA_SHAPE_WHOLE && ((ldd * out_size) % 16 || (C && (ldc * out_size) % 16))) {
     const int epv = 16 / in_size;
-    cls = (layoutA == GZ_ROW_MAJOR && (layoutB == GZ_COL_MAJOR || N % epv == 0)) ? MFMA_SHAPE_RAGGED_MN : MFMA_SHAPE_GENERAL;
+    const bool a_ok = layoutA == GZ_ROW_MAJOR || (layoutB == GZ_ROW_MAJOR && M % epv == 0);
+    cls = (a_ok && (layoutB == GZ_COL_MAJOR || N % epv == 0)) ? MFMA_SHAPE_RAGGED_MN : MFMA_SHAPE_GENERAL;
   }
   return cls;
 }

@@ -1051,6 +1051,19 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
       set_error("mfma rung: no kernel for the transposed problem on this tile");
       return GZ_ERR_UNSUPPORTED;
     }
+    // a column-major A with a row-major B (int8 and the 16-bit types): both operands through the transposing reads
+    if constexpr (!is_fp8(TYPES)) {
+      if constexpr (TILE_256) {
+        if (ring && !akc && !bkc && shape_class == MFMA_SHAPE_RAGGED_MN)
+          GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false, false, false>), ring_lds, StreamK{});
+        if (ring && !akc && !bkc && !edge)
+          GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false, false, false>), ring_lds, StreamK{});
+      }
+      if constexpr (BM == 128 && BN == 128 && WAVES_M == 2 && WAVES_N == 2) {
+        if (ring && !akc && !bkc && !edge)
+          GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false, false, false>), ring_lds, StreamK{});
+      }
+    }
     if constexpr (TILE_256) {
       if (ring && akc && shape_class == MFMA_SHAPE_RAGGED_MN) {
         if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
@@ -1301,7 +1314,7 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
   MfmaCfg cfg = chosen;
   const int edge = mfma_launch_class(cfg, (int)sizeof(in_t), (int)sizeof(typename Traits<TYPES>::out_t), g.M, g.N, g.K,
                                      g.layoutA, g.layoutB, g.A, g.B, g.C, g.D, g.lda, g.ldb, g.ldc, g.ldd);
-  if (adjust) mfma_adjust_general(TYPES, edge, g.layoutA, &cfg);   // launcher's choice: the wave count follows the kernel
+  if (adjust) mfma_adjust_general(TYPES, edge, g.layoutA, g.layoutB, &cfg);   // launcher's choice: the wave count follows the kernel
   switch (cfg.id) {
     case 1: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 0, s);
     case 2: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 0, s);

@@ -35,7 +35,7 @@
 // instruction's first operand: a lane ends up with four consecutive columns of one row of D,
 //     acc[i][j][e] = D(row0 + 16 i + l % 16, col0 + 16 j + 4 (l / 16) + e).
 //
-// K a multiple of the slab (128 bytes), A row-major, B column-major; whole tiles, or (RAGGED) any M and N with
+// K a multiple of the slab (128 bytes); either layout of A and of B (template parameters below); whole tiles, or (RAGGED) any M and N with
 // 16-byte aligned rows.
 #pragma once
 
@@ -126,8 +126,10 @@ template <int ES, int ROW_BYTES> __host__ __device__ constexpr int ring16_row_sw
 // g.M, g.N, g.lda and g.ldb come swapped by the launcher, g.C / g.D / g.ldc / g.ldd are those of the real row-major
 // output.  The MFMAs take their operands in the other order, so that a lane still ends up with four consecutive
 // columns of one row of the real D, and the epilogue walks the accumulator blocks transposed; nothing else changes.
+// A_KC = false: a column-major A (K rows of M contiguous elements) beside a row-major B.  A then takes the route of a
+// row-major B: whole K rows per copy, a K step per copy group, fragments through the transposing LDS reads.
 template <int TYPES, int BM, int BN, int WAVES_M, int WAVES_N, bool RAGGED = false, bool STREAMK = false, bool B_KC = true,
-          bool SWAP = false>
+          bool SWAP = false, bool A_KC = true>
 // (second launch bound: waves per SIMD the registers must leave room for - the 128 x 128 tile, whose five buffers are
 // half the LDS, runs two work-groups per compute unit)
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128) ? 2 : (WAVES_M * WAVES_N) / 4)
@@ -142,13 +144,15 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int NST = 5;              // LDS buffers, one copy group each
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int FM = WM / 16, FN = WN / 16;
-  constexpr int NMMA = FM * FN, NRD = B_KC ? FM + FN : FM + 2 * FN;   // MFMAs and LDS reads per K step
+  constexpr int NRD_A = A_KC ? FM : 2 * FM, NRD_B = B_KC ? FN : 2 * FN;
+  constexpr int NMMA = FM * FN, NRD = NRD_A + NRD_B;   // MFMAs and LDS reads per K step
   constexpr int EPV = 16 / ES;
   constexpr int HK = 64 / ES;         // K rows of a row-major B per copy group: one K step
   constexpr bool F8 = is_fp8(TYPES);
   static_assert(B_KC || !STREAMK, "stream-K with a column-major B only");
   static_assert(!SWAP || !B_KC, "the transposed problem of two column-major operands has a row-major second operand");
   static_assert(!(F8 && STREAMK), "stream-K for int8 and the 16-bit types");
+  static_assert(A_KC || (!B_KC && !SWAP && !STREAMK && !F8), "a column-major A with a row-major B, int8 and the 16-bit types");
   constexpr int A_BYTES = BM / 2 * LINE, B_BYTES = BN / 2 * LINE;
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (8 rows) per wave and group
@@ -229,16 +233,20 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   // lane at LDS position (row, slot) fetching the piece that belongs there (see ring16_row_swizzle)
   constexpr int KRC = 1024 / (BN * ES), LPR = 64 / KRC;
   static_assert(B_KC || (KRC * BN * ES == 1024 && NW * B_PW * KRC == HK), "whole K rows per copy, a K step per group");
-  uint32_t voff_a[2][A_PW], voff_b[B_KC ? 2 : 1][B_PW];
+  constexpr int KRC_A = 1024 / (BM * ES), LPR_A = 64 / KRC_A;
+  static_assert(A_KC || (KRC_A * BM * ES == 1024 && NW * A_PW * KRC_A == HK), "whole K rows per copy, a K step per group");
+  uint32_t voff_a[A_KC ? 2 : 1][A_PW], voff_b[B_KC ? 2 : 1][B_PW];
 #pragma unroll
   for (int par = 0; par < 2; par++) {
+    if constexpr (A_KC) {
 #pragma unroll
-    for (int t = 0; t < A_PW; t++) {
-      // RAGGED: rows past the end are fetched from the last row (an output depends on its own row of A and column
-      // of B only, and those past the end are not stored)
-      int r = 16 * (wave * A_PW + t) + 8 * par + ci;
-      if constexpr (RAGGED) r = min(m0 + r, g.M - 1) - m0;
-      voff_a[par][t] = (uint32_t)((size_t)r * LDA + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+      for (int t = 0; t < A_PW; t++) {
+        // RAGGED: rows past the end are fetched from the last row (an output depends on its own row of A and column
+        // of B only, and those past the end are not stored)
+        int r = 16 * (wave * A_PW + t) + 8 * par + ci;
+        if constexpr (RAGGED) r = min(m0 + r, g.M - 1) - m0;
+        voff_a[par][t] = (uint32_t)((size_t)r * LDA + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+      }
     }
     if constexpr (B_KC) {
 #pragma unroll
@@ -248,6 +256,18 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
         voff_b[par][t] = (uint32_t)((size_t)r * LDB + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
       }
     }
+  }
+  size_t a_group_step = 0;
+  if constexpr (!A_KC) {
+    const int last_piece = (g.M - m0) / EPV - 1;   // RAGGED: M is a multiple of EPV on this path, m0 < M
+#pragma unroll
+    for (int t = 0; t < A_PW; t++) {
+      const int kr = (wave * A_PW + t) * KRC_A + lane / LPR_A;   // K row within the group
+      int piece = (lane % LPR_A) ^ ring16_row_swizzle<ES, BM * ES>(kr);
+      if constexpr (RAGGED) piece = min(piece, last_piece);      // rows past the end: the last piece (not stored)
+      voff_a[0][t] = (uint32_t)((size_t)kr * LDA + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+    }
+    a_group_step = (size_t)HK * LDA;
   }
   size_t b_group_step = 0;
   if constexpr (!B_KC) {
@@ -264,14 +284,18 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   // scalar bases of a tile: its first row of A (first column of a K-contiguous B) at the first K byte of this run; a
   // row-major B's first K row of the run at the tile's first column
   auto a_base_of = [&](int m_first) -> const char* {
-    return reinterpret_cast<const char*>(g.A) + (size_t)m_first * LDA + k_byte0 - COPY_BIAS;
+    if constexpr (A_KC) return reinterpret_cast<const char*>(g.A) + (size_t)m_first * LDA + k_byte0 - COPY_BIAS;
+    else return reinterpret_cast<const char*>(g.A) + (size_t)(2 * slab0) * HK * LDA + (size_t)m_first * ES - COPY_BIAS;
   };
   auto b_base_of = [&](int n_first) -> const char* {
     if constexpr (B_KC) return reinterpret_cast<const char*>(g.B) + (size_t)n_first * LDB + k_byte0 - COPY_BIAS;
     else return reinterpret_cast<const char*>(g.B) + (size_t)(2 * slab0) * HK * LDB + (size_t)n_first * ES - COPY_BIAS;
   };
   // where copy group C of a tile starts, from the tile's bases
-  auto a_group = [&](const char* a_tile, int c) -> const char* { return a_tile + (size_t)(c >> 1) * LINE; };
+  auto a_group = [&](const char* a_tile, int c) -> const char* {
+    if constexpr (A_KC) return a_tile + (size_t)(c >> 1) * LINE;
+    else return a_tile + (size_t)c * a_group_step;
+  };
   auto b_group = [&](const char* b_tile, int c) -> const char* {
     if constexpr (B_KC) return b_tile + (size_t)(c >> 1) * LINE;
     else return b_tile + (size_t)c * b_group_step;
@@ -282,7 +306,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   auto copy_b_begin = [&](int st) { asm_set_m0(m0_b + st * STAGE_BYTES); };
   auto copy_a = [&](auto t_c, auto p_c, const char* src) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - A_PW / 2) * 1024;
-    asm_copy16<OFF>(voff_a[P][Tn], src);
+    asm_copy16<OFF>(voff_a[A_KC ? P : 0][Tn], src);
   };
   auto copy_b = [&](auto t_c, auto p_c, const char* src) {
     constexpr int Tn = decltype(t_c)::value, P = decltype(p_c)::value, OFF = (Tn - B_PW / 2) * 1024;
@@ -297,14 +321,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   // of l / 16 swapped they read neighbouring pieces, which never meet (counter 0 on four waves).
   const int fp = (lane >> 3) & 1, fi = lane & 7;
   const int quarter = ((lane >> 5) & 1) | (((lane >> 4) & 1) << 1);
-  uint32_t a_addr[NST][2], b_addr[NST][B_KC ? 2 : 1];   // row-major B: per buffer, the wave's first 16-column block
+  uint32_t a_addr[NST][A_KC ? 2 : 1], b_addr[NST][B_KC ? 2 : 1];   // transposing reads: per buffer, the wave's first 16-wide block
 #pragma unroll
   for (int jr = 0; jr < NST; jr++) {
     const int buf = (2 * jr + fp) % NST;
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
       const int pos = ((ks * 4 + quarter) ^ fi ^ fp) * 16;
-      a_addr[jr][ks] = lds_base + buf * STAGE_BYTES + (wm * WM / 16) * 1024 + fi * LINE + pos;
+      if constexpr (A_KC) a_addr[jr][ks] = lds_base + buf * STAGE_BYTES + (wm * WM / 16) * 1024 + fi * LINE + pos;
       if constexpr (B_KC) b_addr[jr][ks] = lds_base + buf * STAGE_BYTES + A_BYTES + (wn * WN / 16) * 1024 + fi * LINE + pos;
     }
   }
@@ -335,6 +359,22 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     }
   }
   constexpr int TR_BLOCK_XOR = 16 * ES;   // 16 columns = 16 ES bytes of a K row: one piece of 8-bit, two of 16-bit elements
+  // a column-major A the same way: K rows of BM elements at the start of each buffer
+  constexpr int TR_PITCH_A = BM * ES, TR_R_OFF_A = (16 / TR_LPR) * TR_PITCH_A;
+  if constexpr (!A_KC) {
+    static_assert(A_KC || (WM % 64 == 0 && FM * 16 * ES / 16 <= 16 && (TR_PITCH_A & (TR_PITCH_A - 1)) == 0 &&
+                           STAGE_BYTES % TR_PITCH_A == 0 && TR_R_OFF_A < 65536), "block addresses differ by an exclusive-or");
+    const int i16 = lane & 15, ti = i16 / TR_LPR;
+    const int m_sub = (i16 % TR_LPR) * (8 / ES);
+    const int krow = quarter * (2 * 16 / TR_LPR) + ti;
+    const int f = ring16_row_swizzle<ES, BM * ES>(krow);
+#pragma unroll
+    for (int st = 0; st < NST; st++) {
+      const int m_local = wm * WM + m_sub;
+      const int piece = (m_local / EPV) ^ f;
+      a_addr[st][0] = lds_base + st * STAGE_BYTES + krow * TR_PITCH_A + piece * 16 + (m_local % EPV) * ES;
+    }
+  }
 
   acc_v acc[FM][FN];
 #pragma unroll
@@ -350,14 +390,21 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   asm volatile("s_nop 7" ::: "memory");
   u32x4_t af[2][FM], bf[2][FN];  // register sets of fragments: one per K step of a slab
   u32x2_t bh[2][B_KC ? 1 : FN][2];  // row-major B: the two halves of a fragment as they come out of the transposing reads
+  u32x2_t ah[2][A_KC ? 1 : FM][2];  // column-major A: the same
 
   // 16 rows of a fragment are one 1 KiB row group
   auto read_one = [&](auto set_c, auto r_c, auto jr_c) {
     constexpr int SET = decltype(set_c)::value, R = decltype(r_c)::value, JR = decltype(jr_c)::value;
-    if constexpr (R < FM) asm_ds_read16<R * 1024>(af[SET][R], a_addr[JR][SET]);
-    else if constexpr (B_KC) asm_ds_read16<(R - FM) * 1024>(bf[SET][R - FM], b_addr[JR][SET]);
-    else {  // K step SET of the slab at ring position JR is copy group 2 JR + SET, whole, in its own buffer
-      constexpr int J = (R - FM) / 2, HALF = (R - FM) % 2, ST = (2 * JR + SET) % NST;
+    // (transposing reads: K step SET of the slab at ring position JR is copy group 2 JR + SET, whole, in its own buffer)
+    if constexpr (R < NRD_A) {
+      if constexpr (A_KC) asm_ds_read16<R * 1024>(af[SET][R], a_addr[JR][SET]);
+      else {
+        constexpr int I = R / 2, HALF = R % 2, ST = (2 * JR + SET) % NST;
+        asm_ds_read_tr_x<ES, HALF * TR_R_OFF_A, I * TR_BLOCK_XOR>(ah[SET][I][HALF], a_addr[ST][0]);
+      }
+    } else if constexpr (B_KC) asm_ds_read16<(R - NRD_A) * 1024>(bf[SET][R - NRD_A], b_addr[JR][SET]);
+    else {
+      constexpr int J = (R - NRD_A) / 2, HALF = (R - NRD_A) % 2, ST = (2 * JR + SET) % NST;
       asm_ds_read_tr_x<ES, HALF * TR_R_OFF, J * TR_BLOCK_XOR>(bh[SET][J][HALF], b_addr[ST][0]);
     }
   };
@@ -376,14 +423,23 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     // MFMAs per copy: over the whole step (bf16 4096^3, us: copies over the whole step 97.7, over its first half
     // 99.2, all at its start 104.4)
     constexpr int CPE = NMMA / NCP;
-    constexpr int RDE = (NMMA * 3 / 4) / NRD;          // MFMAs per read: the reads end with the third quarter of the step
-    static_assert(RDE >= 1, "a step's copies are spread evenly over its MFMAs");
+    // MFMAs per read: the reads end with the third quarter of the step (with both operands through the transposing
+    // reads on the small tile there are as many reads as MFMAs: one behind each)
+    constexpr int RDE = (NMMA * 3 / 4) / NRD >= 1 ? (NMMA * 3 / 4) / NRD : 1;
+    static_assert(NRD <= NMMA, "a step's reads fit between its MFMAs");
     asm volatile("s_waitcnt lgkmcnt(0)");
     if constexpr (!B_KC) {
 #pragma unroll
       for (int j = 0; j < FN; j++) {
         asm volatile("" : "+v"(bh[SET][j][0]), "+v"(bh[SET][j][1]));  // after the wait
         bf[SET][j] = u32x4_t{bh[SET][j][0][0], bh[SET][j][0][1], bh[SET][j][1][0], bh[SET][j][1][1]};
+      }
+    }
+    if constexpr (!A_KC) {
+#pragma unroll
+      for (int i = 0; i < FM; i++) {
+        asm volatile("" : "+v"(ah[SET][i][0]), "+v"(ah[SET][i][1]));
+        af[SET][i] = u32x4_t{ah[SET][i][0][0], ah[SET][i][0][1], ah[SET][i][1][0], ah[SET][i][1][1]};
       }
     }
     static_for<NMMA>([&](auto q_c) {
@@ -545,6 +601,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     using ST5 = std::integral_constant<int, (2 * JR + 5) % NST>;
     // a row-major B: a group is a K step's rows, the slab's second group lies a step further
     const char* const b_cp1 = B_KC ? b_cp : b_cp + b_group_step;
+    const char* const a_cp1 = A_KC ? a_cp : a_cp + a_group_step;
     if constexpr (F8) half_f8(I0{}, jr_c, ST4{}, a_cp, b_cp);
     else kstep(I0{}, jr_c, I0{}, ST4{}, a_cp, b_cp);
     if (j + 2 < nslab) {  // the copies of group 2j+4 may stay in flight
@@ -553,10 +610,10 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     } else {
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
-    if constexpr (F8) half_f8(I1{}, jr_c, ST5{}, a_cp, b_cp1);
-    else kstep(I1{}, NEXT{}, I1{}, ST5{}, a_cp, b_cp1);
+    if constexpr (F8) half_f8(I1{}, jr_c, ST5{}, a_cp1, b_cp1);
+    else kstep(I1{}, NEXT{}, I1{}, ST5{}, a_cp1, b_cp1);
     const bool more = j + 3 < nslab;   // the next slab fetches one further
-    a_cp += more ? (size_t)LINE : (size_t)0;
+    a_cp += more ? (A_KC ? (size_t)LINE : 2 * a_group_step) : (size_t)0;
     b_cp += more ? (B_KC ? (size_t)LINE : 2 * b_group_step) : (size_t)0;
   };
 

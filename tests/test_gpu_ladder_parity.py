@@ -162,6 +162,37 @@ def test_whole_line_pipeline_on_the_transposed_problem(G, types):
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.COL, 1, 1)), (types, variant, m, n, k, pads)
 
 
+@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.E4M3E4M3F16))
+def test_whole_line_pipeline_column_major_a_with_row_major_b(G, types):
+    """Neither operand K-contiguous: both go into LDS as whole K rows and come out through the transposing reads
+    (int8 and the 16-bit types; the 8-bit floats run the register-staged kernel on the same calls).  Whole tiles on
+    every variant of the kernel and the launcher's own choice, M and N ragged in whole 16-byte pieces, shapes it
+    cannot take (M = 300), sub-matrix views.  Bit-exact."""
+    slab = 128 // np.dtype(O.IN_DTYPE[types]).itemsize
+    for variant, slabs, (m, n) in itertools.product((0, 5, 6, 9, 10, 11), (1, 2, 5, 6, 11), [(256, 512), (512, 256), (128, 384)]):
+        k = slab * slabs
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs + 40)
+        print("col/row case", types, variant, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.COL, O.ROW, 1, 1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.ROW, 1, 1)), (types, variant, m, n, k)
+    for variant, slabs, (m, n) in itertools.product((0, 5, 6), (1, 4, 7), [(528, 304), (240, 272), (16, 512), (300, 528)]):
+        k = slab * slabs
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs + 20)
+        print("ragged col/row case", types, variant, m, n, k, flush=True)
+        got = G.run_gemm(types, a, b, c, m, n, k, O.COL, O.ROW, 2, -1, MFMA, variant)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.ROW, 2, -1)), (types, variant, m, n, k)
+    piece_in = 16 // np.dtype(O.IN_DTYPE[types]).itemsize
+    piece_out = 16 // np.dtype(O.OUT_DTYPE[types]).itemsize
+    for variant, (m, n), pads in itertools.product((5, 6, 11), [(512, 256), (528, 304)],
+                                                   [(2 * piece_in, piece_in, piece_out, 2 * piece_out), (piece_in, piece_in, 1, 1),
+                                                    (1, 3, piece_out, piece_out)]):
+        k = 3 * slab
+        a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=variant + 5)
+        print("col/row ld case", types, variant, m, n, k, pads, flush=True)
+        got = G.run_gemm_ld(types, a, b, c, m, n, k, O.COL, O.ROW, 1, 1, MFMA, variant, pads)
+        assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.COL, O.ROW, 1, 1)), (types, variant, m, n, k, pads)
+
+
 @pytest.mark.parametrize("types", (O.E4M3E4M3F16, O.E5M2E5M2F16))
 def test_whole_line_pipeline_8bit_floats_on_normal_data(G, types):
     """The 16x16x128 kernel (variants 5 and 6) on N(0,1) data, where every bit of the operands matters: a long K
