@@ -35,8 +35,8 @@
 // instruction's first operand: a lane ends up with four consecutive columns of one row of D,
 //     acc[i][j][e] = D(row0 + 16 i + l % 16, col0 + 16 j + 4 (l / 16) + e).
 //
-// K a multiple of the slab (128 bytes); either layout of A and of B (template parameters below); whole tiles, or (RAGGED) any M and N with
-// 16-byte aligned rows.
+// K a multiple of the slab (128 bytes); either layout of A and of B (template parameters below); whole tiles, or
+// (RAGGED) any M and N with 16-byte aligned lines.
 #pragma once
 
 namespace gz {
