@@ -502,7 +502,8 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
       plan->lds_bytes = mfma_lds_bytes(c);
       plan->grid = (int64_t)ceil_div(m_first, c.bm) * ceil_div(n_first, c.bn);
       // whole tiles on the ring kernel with the 16x16 instructions: one work-group per compute unit walks the tiles
-      if (c.ring == 1 && types != GZ_F32F32F32 && (layoutA == GZ_ROW_MAJOR || (layoutB == GZ_ROW_MAJOR && !is_fp8(types))) &&
+      if (c.ring == 1 && (layoutA == GZ_ROW_MAJOR || (layoutB == GZ_ROW_MAJOR && !is_fp8(types) && types != GZ_F32F32F32)) &&
+          !(types == GZ_F32F32F32 && c.waves_n != 2) &&
           mfma_shape_class(c, es, m_first, n_first, k, layoutA, layoutB) == MFMA_SHAPE_WHOLE)
         plan->grid = mfma_persistent_grid(plan->grid, num_cus);
       if (plan->lds_bytes > lds_per_cu) {

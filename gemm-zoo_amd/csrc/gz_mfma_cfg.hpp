@@ -118,8 +118,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   // a column-major B the launcher runs the transposed problem where it can, see mfma_transposed_ring)
   const bool f8_types = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
   const bool a_direct = a_rows || (!b_cols && !f8_types);
-  const bool ring_ok = a_direct && types != GZ_F32F32F32;
-  const bool ring128_ok = ring_ok && !f8_types;
+  // (fp32: the 256 x 256 tile on four waves with a row-major A)
+  const bool ring_ok = types == GZ_F32F32F32 ? a_rows : a_direct;
+  const bool ring128_ok = ring_ok && !f8_types && types != GZ_F32F32F32;
   const int cand[3] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,
                        ring128_ok ? MFMA_CFG_RING_128 : MFMA_CFG_128};
   double best = 0;
@@ -130,7 +131,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const long long rounds = (tiles + num_cus - 1) / num_cus;
     // whole tiles: every candidate has a direct-to-LDS kernel; ragged M or N: the 256x256 ones only
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
-    const bool direct = a_direct && types != GZ_F32F32F32 &&
+    const bool direct = (types == GZ_F32F32F32 ? a_rows && i == 0 : a_direct) &&
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     // (128 x 128 beyond four rounds: each further round costs a little more, 6144^2 x 6144 = 9 rounds measured
     // 478 us against 457 for three rounds of 256 x 256)
@@ -178,11 +179,12 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // plain estimate; 5000^3, seven, 352 / 307).  The four waves of the 8-bit floats have a large fixed part per tile
     // (epilogue, first slabs: 8000 x 8000 x 1000 46 us a round, 4096 x 4096 x 4000 81), hence the term in 1 / K
     // (8000 x 8000 x 1000, us, 256 x 256 / 256 x 128 / 128 x 128: 181 / 219 / 154).
-    // fp32 has no other kernel, its factor only weighs the splits.
+    // fp32: 2.2 for every kernel (its round against a round of the 16-bit types; it only weighs the splits), a little
+    // less for the hand-scheduled kernel on the 256 x 256 tile.
     const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
     const double staged = f32 ? 2.2 : i == 2 ? 1.05 + 0.05 * (rounds > 4 ? rounds - 4 : 0)
                                     : f8 ? 1.3 + 1000.0 / (double)(K > 0 ? K : 1) : 1.2;
-    const double cost = shape_cost * rowb * (direct ? 1.0 : staged);
+    const double cost = f32 ? shape_cost * (direct ? 0.95 * 2.2 : 2.2) : shape_cost * rowb * (direct ? 1.0 : staged);
     if (i == 0 || cost < best) {
       best = cost;
       pick = cand[i];
@@ -202,7 +204,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
     const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
     bool eight = false;
-    if (f8) {
+    if (types == GZ_F32F32F32) {
+      eight = false;   // one instance: four waves
+    } else if (f8) {
       // 8-bit floats: eight waves up to three rounds of tiles (their 16-bit epilogue has more stores in flight),
       // four beyond.  e4m3, us, four / eight waves, row/row: 4096^3 56.2 / 53.3, 5120^3 122.8 / 115.7, 6144^3
       // 221.5 / 213.0, 4096^2 x 8192 99.6 / 99.0, 8192^3 404.9 / 419.4; row/col 4096^3 53.8 / 50.9, 8192^3
@@ -495,7 +499,7 @@ inline long long mfma_persistent_grid(long long tiles, int num_cus) {
 // the configuration in terms of the transposed problem (bm along N, bn along M).
 inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, int layoutB, int variant, int num_cus,
                                  MfmaCfg* out) {
-  if (layoutA != GZ_COL_MAJOR || layoutB != GZ_COL_MAJOR || types == GZ_F32F32F32 || M <= 0 || N <= 0 || K <= 0) return false;
+  if (layoutA != GZ_COL_MAJOR || layoutB != GZ_COL_MAJOR || M <= 0 || N <= 0 || K <= 0) return false;
   if (variant < 0 || variant > kNumMfmaCfgs) return false;
   if (variant > 0) {
     *out = kMfmaCfgs[variant - 1];
@@ -510,7 +514,8 @@ inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, in
   if (f8 && out->bm != 256) return false;   // the 8-bit floats have the 256 x 256 tile only on that kernel
   // (and their slab schedule wants eight row blocks per wave, which the eight-wave tile laid out the other way round
   // does not have: four waves)
-  if (f8 && out->waves_m * out->waves_n == 8) *out = kMfmaCfgs[out->id - 2];
+  if ((f8 || types == GZ_F32F32F32) && out->waves_m * out->waves_n == 8) *out = kMfmaCfgs[out->id - 2];
+  if (types == GZ_F32F32F32 && out->bm != 256) return false;
   const int cls = mfma_shape_class(*out, mfma_in_size(types), N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR);
   return cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && out->bm == 256);
 }

@@ -142,7 +142,12 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
 // BLK = 16: the accumulators are those of the 16x16 instructions, acc[i][j][e] = D(row0 + 16 i + lane % 16,
 // col0 + 16 j + 4 (lane / 16) + e); FM and FN still count 32-row and 32-column blocks.
 // TRANSPOSED (BLK = 16): the blocks come as acc[j][i], the array of a kernel that ran the transposed problem.
-template <int TYPES, int FM, int FN, bool RAGGED = false, int BLK = 32, bool TRANSPOSED = false, class Acc, int AM, int AN>
+// BY4 (BLK = 16): within a group of 64 columns block 4 g + s holds the columns 4 c + s, c = 0 .. 15, instead of
+// 16 s + c: acc[i][4 g + s][e] = D(row0 + 16 i + lane % 16, col0 + 64 g + 16 (lane / 16) + 4 e + s) - what a kernel
+// ends up with that feeds the matrix instruction four consecutive columns of a row-major B per lane.  A lane's values
+// of the four blocks of a group are then four consecutive columns again.
+template <int TYPES, int FM, int FN, bool RAGGED = false, int BLK = 32, bool TRANSPOSED = false, bool BY4 = false, class Acc,
+          int AM, int AN>
 __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g, Acc (&acc)[AM][AN], int row0, int col0,
                                                        int lane, char* region) {
   static_assert(TRANSPOSED ? (BLK == 16 && AN == FM * 2 && AM == FN * 2)
@@ -159,7 +164,9 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   const int M = g.M, N = g.N;
   const size_t LDC = (size_t)g.ldc, LDD = (size_t)g.ldd;   // elements between the rows of C and of D
   const bool use_c = g.beta != 0;
-  char* wr = BLK == 32 ? region + (lane & 31) * PITCH_E + (lane >> 5) * 16 : region + (lane & 15) * PITCH_E + (lane >> 4) * 16;
+  static_assert(!BY4 || (BLK == 16 && !TRANSPOSED && AN % 4 == 0), "groups of four 16-column blocks");
+  char* wr = BLK == 32 ? region + (lane & 31) * PITCH_E + (lane >> 5) * 16
+                       : region + (lane & 15) * PITCH_E + (lane >> 4) * (BY4 ? 64 : 16);
   const char* rd = region + (lane / LPR) * PITCH_E + (lane % LPR) * W * 4;
   const int n = col0 + (lane % LPR) * W;
   // RAGGED: M or N need not be multiples of the tile and D / C need not be aligned.  Rows and columns past the end
@@ -207,9 +214,16 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         constexpr int H = decltype(h_c)::value;
         static_for<NJ>([&](auto j_c) {
           constexpr int J = decltype(j_c)::value;
-          const Acc& a = acc[TRANSPOSED ? J : 2 * I + H][TRANSPOSED ? 2 * I + H : J];
-          acc_t v[4] = {a[0], a[1], a[2], a[3]};
-          __builtin_memcpy(wr + H * 16 * PITCH_E + J * 64, v, 16);
+          if constexpr (BY4) {   // group J / 4, element J % 4 of its four blocks
+            constexpr int G = J / 4, E = J % 4;
+            acc_t v[4] = {acc[2 * I + H][4 * G + 0][E], acc[2 * I + H][4 * G + 1][E], acc[2 * I + H][4 * G + 2][E],
+                          acc[2 * I + H][4 * G + 3][E]};
+            __builtin_memcpy(wr + H * 16 * PITCH_E + (64 * G + 4 * E) * 4, v, 16);
+          } else {
+            const Acc& a = acc[TRANSPOSED ? J : 2 * I + H][TRANSPOSED ? 2 * I + H : J];
+            acc_t v[4] = {a[0], a[1], a[2], a[3]};
+            __builtin_memcpy(wr + H * 16 * PITCH_E + J * 64, v, 16);
+          }
         });
       });
     }
@@ -1033,6 +1047,26 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
   const size_t dtl_lds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
   const dim3 pgrid((unsigned)(ring == 1 ? mfma_persistent_grid((long long)tiles_m * tiles_n, device_compute_units())
                                         : (long long)tiles_m * tiles_n));
+  // fp32 on the hand-scheduled kernel: the 256 x 256 tile on four waves, a row-major A with either layout of B, and
+  // two column-major operands as the transposed problem (v_mfma_f32_16x16x4_f32, four per block and K step)
+  if constexpr (TYPES == GZ_F32F32F32 && TILE_256 && WAVES_N == 2) {
+    if (transposed) {
+      if (ring && shape_class == MFMA_SHAPE_RAGGED_MN)
+        GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, true, false, false, true>), ring_lds, StreamK{});
+      if (ring && !edge)
+        GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, false, false, false, true>), ring_lds, StreamK{});
+      set_error("mfma rung: no kernel for the transposed problem on this tile");
+      return GZ_ERR_UNSUPPORTED;
+    }
+    if (ring && akc && shape_class == MFMA_SHAPE_RAGGED_MN) {
+      if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
+      else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
+    }
+    if (ring && akc && !edge) {
+      if (bkc) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});
+      else GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
+    }
+  }
   if constexpr (TYPES != GZ_F32F32F32) {
     // `transposed`: g is the transposed problem of a column-major A with a column-major B (see SWAP in
     // rung4_mfma_ring16.hpp), a row-major pair for the ring kernel's operands, with the real C and D

@@ -1,15 +1,16 @@
 // MFMA rung, whole-line ring of five LDS buffers with the 16x16 matrix instructions.
 //
-// Same data movement as mfma_ring5_kernel (whole 128-byte lines per copy, a slab cut by rows into two copy groups,
-// a ring of five 32 KiB buffers, one barrier per slab); what changes is the arithmetic:
-//     v_mfma_f32_16x16x32_{bf16,f16}   v_mfma_i32_16x16x64_i8
-// instead of the 32x32 forms.  A 16x16 instruction sums 64 bytes of K per row inside the matrix pipe before it
+// Data movement: every copy asks the L2 for whole 128-byte lines (8 rows x 128 bytes of K per instruction), so a K
+// slab (128 bytes of K per row) is cut by ROWS into two copy groups; a group fills one of five 32 KiB buffers (all of
+// the LDS), one barrier per slab.  Arithmetic:
+//     v_mfma_f32_16x16x32_{bf16,f16}   v_mfma_i32_16x16x64_i8   v_mfma_f32_16x16x128_f8f6f4
+// rather than the 32x32 forms.  A 16x16 instruction sums 64 bytes of K per row inside the matrix pipe before it
 // touches the accumulators, a 32x32 one 32 bytes, so the same product costs half the accumulator reads and writes -
 // and this part runs against its power limit: an MFMA-only loop on N(0,1) bf16 operands sustains 2100-2130 TFLOPS
 // with the 16x16x32 instruction against 1835-1855 with 32x32x16 (at 2.06 against 1.79 GHz), 1920-1970 against
 // 1710-1735 with the fragment reads of a 256x256 tile interleaved.
 //
-// A K step is then 64 bytes of K per row: a 128-byte slab has two of them, each with (WM / 16) x (WN / 16) MFMAs of
+// A K step is 64 bytes of K per row: a 128-byte slab has two of them, each with (WM / 16) x (WN / 16) MFMAs of
 // 16 cycles and WM / 16 + WN / 16 fragment reads.  Per slab j (groups 2j, 2j+1 in buffers (2j) % 5, (2j+1) % 5):
 //   K step 0 : MFMAs on set 0; requests the fragments of (j, 1) into set 1; issues copy group 2j+4 (A rows, then
 //              B rows) into buffer (2j+4) % 5, which slab j-1 left at its barrier
@@ -21,12 +22,13 @@
 // next step asks for them; its copies are spread evenly over the whole step, one every NMMA / NCP MFMAs: issued as
 // one run behind the reads they cost 1-5 % more (bf16 4096^3 100.5 -> 99.3 us, int8 8192^3 434.5 -> 418.0 on four
 // waves; eight waves at K = 8192: 213.9 -> 198.1).
-// Measured and not taken (bf16 4096^3, four waves, interleaved runs of timing-only builds): no barrier and no wait at
-// all 99.2 against 100.5 us, so nothing waits for data; the copies as plain register loads with no LDS write 106.5
-// against 106.8, so the direct-to-LDS path is not what they cost; all copies from one slab (always L2 hits) 96.5; no
-// copies in the main loop 84.2: the stream from L2 into the compute unit itself holds the matrix pipe at 0.60-0.68
-// busy; a different first slab per tile (so that tiles that share rows do not ask for them at the same moment) lost
-// 1-4 %; copies masked off for three of four waves in turn (exec = 0 is not free) 140 us.
+// What the loop costs is power, not waiting: the copies of a bf16 4096^3 launch alone take 60 us (17.5 TB/s into the
+// compute units), its MFMAs alone 63, both together 77 at a lower clock (bench/probe_operand_stream.cpp), this loop
+// with its fragment reads and barriers 83.  Timing-only builds of this kernel say the same: no barrier and no wait at
+// all 99.2 against 100.5 us for the launch, the copies as plain register loads with no LDS write 106.5 against 106.8,
+// all copies from one slab (always L2 hits) 96.5, no copies in the main loop 84.2; a different first slab per tile
+// (so that tiles that share rows do not ask for them at the same moment) lost 1-4 %; copies switched off by a zero
+// lane mask for three of four waves in turn 140 us (exec = 0 is not free).
 //
 // Fragments: lane l supplies row l % 16 and the 16 bytes of K at piece 4 s + q(l) of K step s, q(l) the two bits of
 // l / 16 swapped (see below); tile row
@@ -51,6 +53,12 @@ __device__ __forceinline__ void asm_mfma16(typename AccVec4<TYPES>::type& c, con
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
   else
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
+}
+// fp32: v_mfma_f32_16x16x4_f32 takes one value per lane and operand, lane l row l % 16 and k = l / 16.  A 16-byte
+// fragment holds four consecutive k of the lane's row: four instructions, each on one register of the two fragments
+// (instruction S sums k = 4 (l / 16) + S over the four lane groups; A and B agree on that, which is all it needs).
+template <int S> __device__ __forceinline__ void asm_mfma16_f32(f32x4_t& c, uint32_t first, uint32_t second) {
+  asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+a"(c) : "v"(first), "v"(second));
 }
 template <int TYPES> __device__ __forceinline__ void asm_touch_acc4(typename AccVec4<TYPES>::type& c) {
   asm volatile("" : "+a"(c));
@@ -86,6 +94,17 @@ template <int ES, int OFF, int XOR> __device__ __forceinline__ void asm_ds_read_
       asm volatile("v_xor_b32 %1, %3, %2\n\tds_read_b64_tr_b8 %0, %1 offset:%4" : "=v"(dst), "=&v"(t) : "v"(addr), "i"(XOR), "i"(OFF));
   }
 }
+// Two 4-byte values, OFF0 and OFF1 times 256 bytes past addr ^ XOR (fp32 fragments of a row-major B: two K rows).
+template <int OFF0, int OFF1, int XOR> __device__ __forceinline__ void asm_ds_read32x2_x(u32x2_t& dst, uint32_t addr) {
+  static_assert(OFF0 >= 0 && OFF0 < 256 && OFF1 >= 0 && OFF1 < 256, "8-bit offsets in units of 64 dwords");
+  if constexpr (XOR == 0) {
+    asm volatile("ds_read2st64_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(dst) : "v"(addr), "i"(OFF0), "i"(OFF1));
+  } else {
+    uint32_t t;
+    asm volatile("v_xor_b32 %1, %3, %2\n\tds_read2st64_b32 %0, %1 offset0:%4 offset1:%5"
+                 : "=v"(dst), "=&v"(t) : "v"(addr), "i"(XOR), "i"(OFF0), "i"(OFF1));
+  }
+}
 __device__ __forceinline__ void asm_touch_v2(u32x2_t& a, u32x2_t& b, u32x2_t& c, u32x2_t& d) {
   asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
@@ -115,9 +134,12 @@ constexpr size_t STREAMK_SLOT_ELEMS = 256 * 256;
 // the two blocks that one half of the wave reads in the same cycle.
 // (Rows of 128 bytes - int8 with a 128-column tile - hold eight pieces, and consecutive rows already lie in different
 // halves of the 64 banks: the row's lowest bit stays out of the swizzle, which then fits three bits.)
+// fp32 has no transposing read: a lane takes one value per K row (two rows per ds_read2st64_b32), sixteen lanes
+// sixteen consecutive columns of it (64 bytes) and the four lane groups K rows four apart, which the swizzle sends
+// 64 bytes apart.
 template <int ES, int ROW_BYTES> __host__ __device__ constexpr int ring16_row_swizzle(int r) {
   static_assert(ROW_BYTES >= 256 || (ES == 1 && ROW_BYTES == 128), "a K row of at least sixteen pieces, or eight of int8");
-  return ES == 2 ? (((r & 3) << 2) ^ (((r >> 3) & 1) << 1))
+  return ES == 4 ? (((r >> 2) & 3) << 2) : ES == 2 ? (((r & 3) << 2) ^ (((r >> 3) & 1) << 1))
                  : ROW_BYTES >= 256 ? (((r & 7) << 1) ^ ((r >> 4) & 1)) : ((((r >> 1) & 3) << 1) ^ ((r >> 4) & 1));
 }
 
@@ -144,7 +166,11 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int NST = 5;              // LDS buffers, one copy group each
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int FM = WM / 16, FN = WN / 16;
-  constexpr int NRD_A = A_KC ? FM : 2 * FM, NRD_B = B_KC ? FN : 2 * FN;
+  constexpr bool F32 = TYPES == GZ_F32F32F32;
+  constexpr int SUB = F32 ? 4 : 1;    // matrix instructions per 16 x 16 block and K step
+  // fp32 with a row-major B (and not the transposed problem): four consecutive COLUMNS per lane, see b4 below
+  constexpr bool B4 = F32 && !B_KC && !SWAP;
+  constexpr int NRD_A = A_KC ? FM : 2 * FM, NRD_B = (B_KC || B4) ? FN : 2 * FN;
   constexpr int NMMA = FM * FN, NRD = NRD_A + NRD_B;   // MFMAs and LDS reads per K step
   constexpr int EPV = 16 / ES;
   constexpr int HK = 64 / ES;         // K rows of a row-major B per copy group: one K step
@@ -157,7 +183,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (8 rows) per wave and group
   constexpr int NCP = A_PW + B_PW;
-  static_assert(TYPES != GZ_F32F32F32, "8- and 16-bit operands");
+  static_assert(!F32 || (BM == 256 && BN == 256 && NW == 4 && A_KC && !STREAMK), "fp32: the 256 x 256 tile on four waves, row-major A");
   static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && NW == 4 && !F8 && !STREAMK),
                 "the 256 x 256 tile, or the 128 x 128 tile on four waves for int8 and the 16-bit types");
   static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile rows must divide over the waves");
@@ -338,7 +364,34 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int TR_LPR = ES == 2 ? 4 : 2;                 // lanes per K row of a block
   constexpr int TR_PITCH = BN * ES;                       // bytes between K rows
   constexpr int TR_R_OFF = (16 / TR_LPR) * TR_PITCH;      // second half of a fragment
-  if constexpr (!B_KC) {
+  if constexpr (B4) {
+    // A 16-byte read of a K row gives a lane four consecutive columns.  Lane group q of read g takes K row 4 q + g
+    // (the k that register g of the A fragment stands for), lane c of the group columns 4 c .. 4 c + 3 of a group
+    // of 64: register s of the read is then a B fragment for the sixteen columns 4 c + s, and the four
+    // instructions on (register g of A, register s of read g) for g = 0 .. 3 sum the sixteen k of the step into
+    // accumulator block 4 G + s of column group G.  One read per four MFMAs' worth of B, as with a K-contiguous B;
+    // the epilogue knows the column order (BY4).
+    static_assert(!B4 || (WN % 64 == 0 && 3 * TR_PITCH + (WN / 64 - 1) * 256 < 65536), "immediate offsets");
+    const int krow = quarter * 4;
+    const int f = ring16_row_swizzle<ES, BN * ES>(krow);
+#pragma unroll
+    for (int st = 0; st < NST; st++) {
+      const int piece = ((wn * WN) / EPV + (lane & 15)) ^ f;
+      b_addr[st][0] = lds_base + st * STAGE_BYTES + A_BYTES + krow * TR_PITCH + piece * 16;
+    }
+  } else if constexpr (!B_KC && F32) {
+    // fp32: lane group q takes K rows 4 q + S (S by the immediate offset), the lane column l % 16 of the block
+    static_assert(!F32 || B_KC || (WN % 64 == 0 && (TR_PITCH & (TR_PITCH - 1)) == 0 && STAGE_BYTES % TR_PITCH == 0 &&
+                                   A_BYTES % TR_PITCH == 0 && 3 * TR_PITCH < 65536), "block addresses differ by an exclusive-or");
+    const int krow = quarter * 4;
+    const int f = ring16_row_swizzle<ES, BN * ES>(krow);   // the same for the four rows of a lane group
+#pragma unroll
+    for (int st = 0; st < NST; st++) {
+      const int n_local = wn * WN + (lane & 15);
+      const int piece = (n_local / EPV) ^ f;
+      b_addr[st][0] = lds_base + st * STAGE_BYTES + A_BYTES + krow * TR_PITCH + piece * 16 + (n_local % EPV) * ES;
+    }
+  } else if constexpr (!B_KC) {
     static_assert(B_KC || TR_R_OFF < 65536, "immediate offset");
     const int i16 = lane & 15, ti = i16 / TR_LPR;
     const int n_sub = (i16 % TR_LPR) * (8 / ES);
@@ -391,6 +444,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   u32x4_t af[2][FM], bf[2][FN];  // register sets of fragments: one per K step of a slab
   u32x2_t bh[2][B_KC ? 1 : FN][2];  // row-major B: the two halves of a fragment as they come out of the transposing reads
   u32x2_t ah[2][A_KC ? 1 : FM][2];  // column-major A: the same
+  u32x2_t bq[2][(F32 && !B_KC && !B4) ? FN : 1][2];   // fp32, transposed problem: a fragment's four values, two K rows per read
+  u32x4_t b4[2][B4 ? FN / 4 : 1][4];                  // fp32, row-major B: [column group][read g], four columns each
 
   // 16 rows of a fragment are one 1 KiB row group
   auto read_one = [&](auto set_c, auto r_c, auto jr_c) {
@@ -403,7 +458,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
         asm_ds_read_tr_x<ES, HALF * TR_R_OFF_A, I * TR_BLOCK_XOR>(ah[SET][I][HALF], a_addr[ST][0]);
       }
     } else if constexpr (B_KC) asm_ds_read16<(R - NRD_A) * 1024>(bf[SET][R - NRD_A], b_addr[JR][SET]);
-    else {
+    else if constexpr (B4) {
+      constexpr int G = (R - NRD_A) / 4, RG = (R - NRD_A) % 4, ST = (2 * JR + SET) % NST;
+      asm_ds_read16<RG * TR_PITCH + G * 256>(b4[SET][G][RG], b_addr[ST][0]);
+    } else if constexpr (F32) {
+      constexpr int J = (R - NRD_A) / 2, HALF = (R - NRD_A) % 2, ST = (2 * JR + SET) % NST;
+      static_assert(!F32 || B_KC || TR_PITCH % 256 == 0, "K rows whole units of the two-address read apart");
+      asm_ds_read32x2_x<2 * HALF * (TR_PITCH / 256), (2 * HALF + 1) * (TR_PITCH / 256), J * TR_BLOCK_XOR>(bq[SET][J][HALF], b_addr[ST][0]);
+    } else {
       constexpr int J = (R - NRD_A) / 2, HALF = (R - NRD_A) % 2, ST = (2 * JR + SET) % NST;
       asm_ds_read_tr_x<ES, HALF * TR_R_OFF, J * TR_BLOCK_XOR>(bh[SET][J][HALF], b_addr[ST][0]);
     }
@@ -422,13 +484,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
     constexpr int SET = decltype(set_c)::value, CST = decltype(cst_c)::value;
     // MFMAs per copy: over the whole step (bf16 4096^3, us: copies over the whole step 97.7, over its first half
     // 99.2, all at its start 104.4)
-    constexpr int CPE = NMMA / NCP;
+    constexpr int CPE = NMMA * SUB / NCP;
     // MFMAs per read: the reads end with the third quarter of the step (with both operands through the transposing
     // reads on the small tile there are as many reads as MFMAs: one behind each)
-    constexpr int RDE = (NMMA * 3 / 4) / NRD >= 1 ? (NMMA * 3 / 4) / NRD : 1;
-    static_assert(NRD <= NMMA, "a step's reads fit between its MFMAs");
+    constexpr int RDE = (NMMA * SUB * 3 / 4) / NRD >= 1 ? (NMMA * SUB * 3 / 4) / NRD : 1;
+    static_assert(NRD <= NMMA * SUB, "a step's reads fit between its MFMAs");
     asm volatile("s_waitcnt lgkmcnt(0)");
-    if constexpr (!B_KC) {
+    if constexpr (!B_KC && !F32) {
 #pragma unroll
       for (int j = 0; j < FN; j++) {
         asm volatile("" : "+v"(bh[SET][j][0]), "+v"(bh[SET][j][1]));  // after the wait
@@ -442,10 +504,17 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
         af[SET][i] = u32x4_t{ah[SET][i][0][0], ah[SET][i][0][1], ah[SET][i][1][0], ah[SET][i][1][1]};
       }
     }
-    static_for<NMMA>([&](auto q_c) {
-      constexpr int Q = decltype(q_c)::value;
-      constexpr int I = Q / FN, J = (I & 1) ? FN - 1 - Q % FN : Q % FN;
-      if constexpr (SWAP) asm_mfma16<TYPES>(acc[I][J], af[SET][I], bf[SET][J]);
+    // (fp32: four sweeps over the blocks, one per register of the fragments, so that the four instructions of a block
+    // lie NMMA instructions apart and none waits for the one before on the same accumulators)
+    static_for<NMMA * SUB>([&](auto q_c) {
+      constexpr int Q = decltype(q_c)::value, S = Q / NMMA, QB = Q % NMMA;
+      constexpr int I = QB / FN, J = (I & 1) ? FN - 1 - QB % FN : QB % FN;
+      if constexpr (F32) {
+        if constexpr (B_KC) asm_mfma16_f32<S>(acc[I][J], bf[SET][J][S], af[SET][I][S]);
+        else if constexpr (B4) asm_mfma16_f32<S>(acc[I][J], b4[SET][J / 4][S][J % 4], af[SET][I][S]);
+        else if constexpr (SWAP) asm_mfma16_f32<S>(acc[I][J], af[SET][I][S], bq[SET][J][S / 2][S % 2]);
+        else asm_mfma16_f32<S>(acc[I][J], bq[SET][J][S / 2][S % 2], af[SET][I][S]);
+      } else if constexpr (SWAP) asm_mfma16<TYPES>(acc[I][J], af[SET][I], bf[SET][J]);
       else asm_mfma16<TYPES>(acc[I][J], bf[SET][J], af[SET][I]);
       if constexpr (Q % RDE == RDE - 1 && Q / RDE < NRD)
         read_one(std::integral_constant<int, SET ^ 1>{}, std::integral_constant<int, Q / RDE>{}, rj_c);
@@ -681,8 +750,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
       gr.N = g.M;
       store_accumulators_lds<TYPES, WN / 32, WM / 32, RAGGED, 16, true>(gr, acc, n0 + wn * WN, m0 + wm * WM, lane, staging);
     } else {
-      store_accumulators_lds<TYPES, WM / 32, WN / 32, RAGGED, 16>(g, acc, m0 + wm * WM, n0 + wn * WN, lane,
-                                                                  staging);
+      store_accumulators_lds<TYPES, WM / 32, WN / 32, RAGGED, 16, false, B4>(g, acc, m0 + wm * WM, n0 + wn * WN, lane,
+                                                                            staging);
     }
     if constexpr (!PERSISTENT) break;
     bid += (int)gridDim.x;

@@ -93,14 +93,15 @@ def test_edge_tiles_of_the_register_staged_kernel(G, types):
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, la, lb, 1, 1)), (types, variant, la, lb, m, n, k)
 
 
-@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.E4M3E4M3F16, O.E5M2E5M2F16))
+@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.E4M3E4M3F16, O.E5M2E5M2F16,
+                                   O.F32F32F32))
 def test_whole_line_pipeline_every_slab_count(G, types):
     """Whole 256x256 tiles, row-major A, column-major B, K = 1..12 slabs of 128 bytes: the kernel whose ring of five
     buffers is filled by whole-line copies (variants 5 and 6; 9 and 10 launch one work-group per tile), through a full
     turn of the ring and past it."""
     slab = 128 // np.dtype(O.IN_DTYPE[types]).itemsize
     # (variant 11: the same kernel on 128 x 128 tiles; the 8-bit floats have no such instance and run the tile's
-    # register-staged kernel)
+    # register-staged kernel; fp32 has the four-wave 256 x 256 instances only - v_mfma_f32_16x16x4_f32, four per block)
     for variant, slabs, (m, n) in itertools.product((5, 6, 9, 10, 11), (1, 2, 3, 4, 5, 6, 7, 9, 10, 11, 12), [(256, 512), (512, 256)]):
         k = slab * slabs
         a, b, c = O.make_inputs(types, m, n, k, kind=exact_kind(types), seed=slabs)
@@ -130,7 +131,8 @@ def test_whole_line_pipeline_every_slab_count(G, types):
         assert np.array_equal(got, O.gemm(types, a, b, c, m, n, k, O.ROW, O.ROW, 1, 1)), (types, variant, m, n, k)
 
 
-@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.E4M3E4M3F16, O.E5M2E5M2F16))
+@pytest.mark.parametrize("types", (O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.E4M3E4M3F16, O.E5M2E5M2F16,
+                                   O.F32F32F32))
 def test_whole_line_pipeline_on_the_transposed_problem(G, types):
     """Column-major A and B: the same kernel runs D^T = B^T A^T (a row-major pair of operands) and writes the
     row-major D.  Whole tiles on every variant of that kernel, the launcher's own choice, M and N ragged (M in whole
