@@ -422,7 +422,8 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         plan->grid = (int64_t)ceil_div(m, 128) * ceil_div(n, 128);
         return GZ_OK;
       }
-      if (MfmaCfg ct; mfma_transposed_ring(types, m, n, k, layoutA, layoutB, variant, num_cus, &ct)) {
+      MfmaSplit tsp;
+      if (MfmaCfg ct; mfma_transposed_ring(types, m, n, k, layoutA, layoutB, variant, num_cus, &ct, &tsp)) {
         // column-major A and B: the ring kernel on the transposed problem (as launch_mfma, aligned operands assumed);
         // the configuration's rows run along N there
         plan->variant = ct.id;
@@ -430,9 +431,16 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         plan->wave_m = ct.bn / ct.waves_m; plan->wave_n = ct.bm / ct.waves_n;
         plan->threads = ct.waves_m * ct.waves_n * 64;
         plan->lds_bytes = mfma_lds_bytes(ct);
-        plan->grid = (int64_t)ceil_div(n, ct.bm) * ceil_div(m, ct.bn);
-        if (ct.ring == 1 && mfma_shape_class(ct, es, n, m, k, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE)
+        const int n_first = tsp.rows_main > 0 ? tsp.rows_main : n;   // columns of the first launch
+        plan->grid = (int64_t)ceil_div(n_first, ct.bm) * ceil_div(m, ct.bn);
+        if (ct.ring == 1 && mfma_shape_class(ct, es, n_first, m, k, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE)
           plan->grid = mfma_persistent_grid(plan->grid, num_cus);
+        if (tsp.rows_main > 0) {   // the remaining columns in a second launch
+          plan->tail_cols = n - tsp.rows_main;
+          plan->tail_tile_m = tsp.tail.bn;
+          plan->tail_tile_n = tsp.tail.bm;
+          plan->tail_grid = (int64_t)ceil_div(n - tsp.rows_main, tsp.tail.bm) * ceil_div(m, tsp.tail.bn);
+        }
         if (plan->lds_bytes > lds_per_cu) {
           set_error("mfma variant %d needs %d bytes of LDS, device has %d", ct.id, plan->lds_bytes, lds_per_cu);
           return GZ_ERR_UNSUPPORTED;
@@ -492,7 +500,8 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
       }
       if (variant == 0) {   // as the launcher does, with 16-byte aligned operands assumed
         int cls = mfma_shape_class(c, es, m_first, n_first, k, layoutA, layoutB);
-        if (plan->tail_cols && layoutB == GZ_ROW_MAJOR) cls = MFMA_SHAPE_GENERAL;
+        // (a column range of a row-major B keeps the pitch of the whole matrix: whole 16-byte pieces or not)
+        if (plan->tail_cols && layoutB == GZ_ROW_MAJOR && ((int64_t)n * es) % 16 != 0) cls = MFMA_SHAPE_GENERAL;
         mfma_adjust_general(types, cls, layoutA, layoutB, &c);
       }
       plan->variant = c.id;

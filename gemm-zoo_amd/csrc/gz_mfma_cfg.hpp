@@ -152,7 +152,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // (the ring kernel: 0.72 of a round up to half a round of tiles, rising to a whole one - 4352 x 4096, 16 tiles
       // left, 0.76; 6144^2, 64, 0.69; 5120^2, 144, 0.74; 5632^2, 228, 0.99)
       if (direct && rem) shape_cost = (double)full + 0.72 + (frac > 0.5 ? 0.56 * (frac - 0.5) : 0.0);
-      if (direct && full == 0) shape_cost = 0.85;
+      // below one round (on eight waves, which such a grid gets): 0.77 up to half a round of tiles, rising to a
+      // whole one (bf16 K = 4096, us: 81 tiles 74, 128 75, 144 78, 160 80, 192 88 against 97 for 256)
+      if (direct && full == 0) shape_cost = 0.77 + (frac > 0.5 ? 0.46 * (frac - 0.5) : 0.0);
     }
     // fp32 is bound by its matrix rate at every tile size, so a smaller tile costs what its share of the products
     // costs: 256 x 128 half a round per round of its own, 128 x 128 its tiles over four per compute unit (measured,
@@ -166,6 +168,24 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     if (i == 2 && direct && ring128_ok) {
       const long long full2 = tiles / (2LL * num_cus), rem2 = tiles % (2LL * num_cus);
       shape_cost = 0.66 * full2 + (rem2 ? 0.36 + 0.15 * (double)rem2 / num_cus : 0.0);
+    }
+    // 128 x 128 tiles on the register-staged kernel (ragged M / N, K-contiguous B), up to three rounds: measured in
+    // rounds of 256 x 256, bf16 K = 4096 - 324 tiles 0.70, 504 0.81, 512 0.80, 576 1.09, 640 1.11, 768 1.19 (the line
+    // below said 0.99 for the first three and 1.27 for the others, and 2300^2 x 4096 ran 256 x 256 tiles in 82 us
+    // instead of these in 67)
+    bool fitted128 = false;
+    if (i == 2 && !direct && !f32 && tiles <= 3LL * num_cus) {
+      shape_cost = tiles <= 2LL * num_cus ? 0.50 + 0.30 * (double)tiles / (2.0 * num_cus)
+                                          : 1.06 + 0.13 * (double)(tiles - 2LL * num_cus) / num_cus;
+      // Against a grid of 256 x 256 tiles below one round these start and end faster and cost more per slab (512
+      // tiles against 128 of 256 x 256, ragged, bf16, us: K = 2048 41.5 / 45.8, K = 4096 75.0 / 74.9 - lines of
+      // 8 + 1.03 per slab and 16.7 + 0.91 per slab); the figures above are those of K = 4096.
+      if (tiles <= 2LL * num_cus) {
+        const double nslab = (double)K * in_size / MFMA_SLAB_BYTES;
+        double kf = (8.0 + 1.03 * nslab) / (16.7 + 0.91 * nslab) / 0.987;
+        shape_cost *= kf < 0.88 ? 0.88 : kf > 1.06 ? 1.06 : kf;
+      }
+      fitted128 = true;
     }
     if (f32 && i == 1) shape_cost = 0.52 * rounds;
     if (f32 && i == 2) shape_cost = 0.10 + 1.15 * (double)tiles / (4.0 * num_cus);
@@ -184,7 +204,8 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
     const double staged = f32 ? 2.2 : i == 2 ? 1.05 + 0.05 * (rounds > 4 ? rounds - 4 : 0)
                                     : f8 ? 1.3 + 1000.0 / (double)(K > 0 ? K : 1) : 1.2;
-    const double cost = f32 ? shape_cost * (direct ? 0.95 * 2.2 : 2.2) : shape_cost * rowb * (direct ? 1.0 : staged);
+    const double cost = f32 ? shape_cost * (direct ? 0.95 * 2.2 : 2.2)
+                            : shape_cost * rowb * (direct || fitted128 ? 1.0 : staged);
     if (i == 0 || cost < best) {
       best = cost;
       pick = cand[i];
@@ -192,12 +213,14 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   }
   *out = kMfmaCfgs[pick];
   if (pick == MFMA_CFG_RING_128) {
-    // A K-contiguous B while every work-group has a compute unit to itself: the register-staged kernel, whose plain
-    // loads get a little more out of a lone work-group's path to the L2 (us, ring / register-staged, bf16 cubes:
-    // 1024 13.5 / 13.3, 1536 21.8 / 19.3, 2048 27.8 / 25.6; two per compute unit: 2560 39.0 / 44.5).  A row-major B
-    // always the ring (1024 13.8 / 18.6, 2048 27.9 / 39.9; int8 1024^3 9.3 / 10.9).
+    // A K-contiguous B on a grid that leaves a good third of the compute units idle: the register-staged kernel,
+    // whose plain loads get as much out of a lone work-group's path to the L2 and which starts a little faster (us,
+    // ring / register-staged, K = 4096: int8 1024^2 19.2 / 18.6, 1536^2 19.7 / 18.9; f16 33.2 / 32.5, 33.9 / 33.2;
+    // bf16 -> f32 33.4 / 34.9, 33.8 / 35.3).  With every compute unit busy the ring (2048^2, 256 tiles: int8
+    // 21.1 / 23.1, f16 37.1 / 42.9, bf16 35.7 / 41.3; K = 1024: 9.6 / 9.7, 13.5 / 14.5, 13.1 / 14.1), as for a
+    // row-major B at every size (1024 13.8 / 18.6, 2048 27.9 / 39.9; int8 1024^3 9.3 / 10.9).
     const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
-    if (b_cols && tiles <= num_cus) *out = kMfmaCfgs[MFMA_CFG_128];
+    if (b_cols && types != GZ_BF16BF16F32 && tiles <= num_cus * 5LL / 8) *out = kMfmaCfgs[MFMA_CFG_128];
   }
   if (pick == MFMA_CFG_RING_W4) {
     // Waves per 256 x 256 tile on the ring kernel.
@@ -228,6 +251,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // bf16 -> f32 row/row: 4096^2 35.1 / 36.5, 101.5 / 101.2; 5120^2 61.7 / 58.7, 175.8 / 173.6; 8192^2
       // 154.2 / 155.9, 398.2 / 415.6; int8 row/col 4096^2 24.1 / 25.3, 55.2 / 58.6; 5120^2 42.1 / 38.4, 94.4 / 94.2;
       // 8192^2 106.0 / 106.2, 231.6 / 248.9.
+      // (a column-major A beside a row-major B: both operands through the transposing reads, two per fragment, which
+      // four waves cannot fit between their MFMAs - eight at every size: bf16 4096^3 101 / 98 us, 5120^2 x 4096
+      // 188 / 174, 7168^2 x 4096 377 / 356, 8000 x 1000 x 4096 94 / 76)
       const bool out16 = types == GZ_BF16BF16BF16 || types == GZ_F16F16F16;
       const double nslab = (double)K * in_size / MFMA_SLAB_BYTES;
       const bool under_a_round = tiles < num_cus, whole_rounds = tiles % num_cus == 0;
@@ -236,7 +262,10 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       if (tiles >= 3LL * num_cus) slope8 *= 1.05;   // past three rounds four waves pull ahead (8192^2 x 4096 above)
       const double fixed4 = out16 ? 13.6 : 13.2;
       const double fixed8 = out16 ? 9.6 : whole_rounds ? 14.1 : 10.5;   // compute units left empty: more of the power and of the L2 for the busy ones
-      eight = fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
+      // Below one round: eight.  With half the compute units idle the busy ones are not held by power, the slopes are
+      // the same and eight waves' fixed part is 8 us lower (about 140 tiles, us, four / eight waves, K = 2048 and 4096:
+      // row/col 54.3 / 46.0, 86.7 / 78.2; row/row 55.3 / 46.0, 89.3 / 77.6; whole tiles, 3072^2: 79.1 / 76.6, 80.5 / 73.7).
+      eight = !a_rows || under_a_round || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
     }
     if (eight) *out = kMfmaCfgs[MFMA_CFG_RING_W8];
   }
@@ -294,6 +323,10 @@ inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int 
   const long long tiles_n = (N + 255) / 256, tiles_m = (M + 255) / 256;
   const long long full = tiles_m * tiles_n / num_cus * num_cus;   // tiles in whole rounds
   if (full == 0 || full == tiles_m * tiles_n) return false;
+  // Only where few tiles remain: the ring kernel's persistent launch carries a larger remainder better than a second
+  // launch does (5120^2 x 4096, 144 of 400 tiles remain, us, one launch / two: bf16 167.7 / 170.3, row-major B
+  // 170.2 / 176.9, int8 95.2 / 99.5; with 16 remaining the cut wins: 4352 x 4096^2 row/row 149 / 141, 7168^2 355 / 338).
+  if (tiles_m * tiles_n - full > num_cus / 4) return false;
   const long long tile_rows = full / tiles_n;                     // tile rows that fit them
   if (tile_rows <= 0 || tile_rows * 256 >= M) return false;
   const int rows_main = (int)(tile_rows * 256);
@@ -339,11 +372,15 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   const int cols_main = N - r;
   MfmaCfg main_cfg, tail_cfg;
   double cost_main = mfma_choose(types, M, cols_main, K, layoutA, layoutB, num_cus, &main_cfg);
-  // the first launch keeps a direct-to-LDS kernel only with row-major A, K-contiguous B and a 256 x 256 tile
+  // the first launch keeps the ring kernel on a 256 x 256 tile where the layouts allow it and the rows of a
+  // row-major B, which keep the pitch of the whole matrix, are whole 16-byte pieces
   const int cls = mfma_shape_class(main_cfg, mfma_in_size(types), M, cols_main, K, layoutA, layoutB);
-  const bool direct_before = layoutA == GZ_ROW_MAJOR && types != GZ_F32F32F32 &&
+  const bool f8_types = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
+  const bool layouts_ok = layoutA == GZ_ROW_MAJOR || (layoutB == GZ_ROW_MAJOR && !f8_types);
+  const bool direct_before = layouts_ok && types != GZ_F32F32F32 &&
                              (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && main_cfg.bm == 256 && main_cfg.bn == 256));
-  const bool direct_after = direct_before && layoutB == GZ_COL_MAJOR && main_cfg.bm == 256 && main_cfg.bn == 256;
+  const bool direct_after = direct_before && main_cfg.bm == 256 && main_cfg.bn == 256 &&
+                            (layoutB == GZ_COL_MAJOR || ((long long)N * mfma_in_size(types)) % 16 == 0);
   if (direct_before && !direct_after) cost_main *= types == GZ_F32F32F32 ? 2.2 : mfma_in_size(types) == 2 ? 1.2 : 1.5;
   // on the register-staged kernel eight waves carry a 256 x 256 tile of 16-bit elements better than four
   // (fp16 4095 x 4097 x 1023, row-major B: 119 us against 158)
@@ -497,17 +534,28 @@ inline long long mfma_persistent_grid(long long tiles, int num_cus) {
 // problem - the launcher's own choice for it is that kernel and neither a cut nor stream-K, or the caller names a
 // variant of the ring kernel - and its tiles are whole (or ragged in M / N on the 256 x 256 tile).  Fills `out` with
 // the configuration in terms of the transposed problem (bm along N, bn along M).
+// `split`, if given: a row cut of the transposed problem (columns of the real one) where the launcher would make one and
+// both parts run the ring kernel; rows_main = 0 otherwise.
 inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, int layoutB, int variant, int num_cus,
-                                 MfmaCfg* out) {
+                                 MfmaCfg* out, MfmaSplit* split = nullptr) {
+  if (split) split->rows_main = 0;
   if (layoutA != GZ_COL_MAJOR || layoutB != GZ_COL_MAJOR || M <= 0 || N <= 0 || K <= 0) return false;
   if (variant < 0 || variant > kNumMfmaCfgs) return false;
   if (variant > 0) {
     *out = kMfmaCfgs[variant - 1];
   } else {
-    MfmaSplit sp;
-    MfmaColSplit cs;
-    if (mfma_resolve_cut(types, N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, &sp, &cs) != 0) return false;
     (void)mfma_choose(types, N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, out);
+    MfmaSplit sp;
+    const int in_size = mfma_in_size(types);
+    auto whole = [&](const MfmaCfg& c, int rows) {
+      return c.ring != 0 && !c.stream_k && mfma_shape_class(c, in_size, rows, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE;
+    };
+    if (split && types != GZ_F32F32F32 && types != GZ_E4M3E4M3F16 && types != GZ_E5M2E5M2F16 &&
+        mfma_resolve_split(types, N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, &sp) && whole(sp.main, sp.rows_main) &&
+        whole(sp.tail, N - sp.rows_main)) {
+      *split = sp;
+      *out = sp.main;
+    }
   }
   if (out->ring == 0 || out->stream_k) return false;
   const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;

@@ -1401,15 +1401,35 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
   GemmArgs<TYPES> g = args;
   const int num_cus = device_compute_units();
   g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), num_cus);
-  // Column-major A and B: the transposed problem on the ring kernel, where one launch of it covers the problem
-  if (MfmaCfg ct; mfma_transposed_ring(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, num_cus, &ct)) {
+  // Column-major A and B: the transposed problem on the ring kernel - one launch, or where the launcher would cut
+  // the rows of the transposed problem (a mostly empty last round) two, over column ranges of the real C and D
+  MfmaSplit tsp;
+  if (MfmaCfg ct; mfma_transposed_ring(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, num_cus, &ct, &tsp)) {
     GemmArgs<TYPES> t = g;
     t.A = g.B; t.B = g.A;
     t.M = g.N; t.N = g.M;
     t.lda = g.ldb; t.ldb = g.lda;
     t.layoutA = GZ_ROW_MAJOR; t.layoutB = GZ_ROW_MAJOR;
-    const int cls = mfma_launch_class(ct, (int)sizeof(typename Traits<TYPES>::in_t), (int)sizeof(typename Traits<TYPES>::out_t),
-                                      t.M, t.N, t.K, t.layoutA, t.layoutB, t.A, t.B, t.C, t.D, t.lda, t.ldb, t.ldc, t.ldd);
+    auto cls_of = [&](const GemmArgs<TYPES>& a, const MfmaCfg& c) {
+      return mfma_launch_class(c, (int)sizeof(typename Traits<TYPES>::in_t), (int)sizeof(typename Traits<TYPES>::out_t), a.M, a.N,
+                               a.K, a.layoutA, a.layoutB, a.A, a.B, a.C, a.D, a.lda, a.ldb, a.ldc, a.ldd);
+    };
+    if (tsp.rows_main > 0) {
+      GemmArgs<TYPES> top = t, bottom = t;
+      top.M = tsp.rows_main;
+      bottom.M = t.M - tsp.rows_main;
+      bottom.A = t.A + (size_t)tsp.rows_main * (size_t)t.lda;   // rows of the transposed problem: columns of B, C and D
+      if (t.C) bottom.C = t.C + tsp.rows_main;
+      bottom.D = t.D + tsp.rows_main;
+      if (cls_of(top, tsp.main) == MFMA_SHAPE_WHOLE && cls_of(bottom, tsp.tail) == MFMA_SHAPE_WHOLE) {
+        const int st = launch_one<TYPES>(top, tsp.main, s, false, true);
+        if (st != GZ_OK) return st;
+        return launch_one<TYPES>(bottom, tsp.tail, s, false, true);
+      }
+      (void)mfma_choose(TYPES, t.M, t.N, t.K, t.layoutA, t.layoutB, num_cus, &ct);   // odd pitches: one launch
+      if (ct.ring == 0) ct = kMfmaCfgs[MFMA_CFG_RING_W4];
+    }
+    const int cls = cls_of(t, ct);
     // (unaligned operands, or rows of D that are not: the kernels of the problem as given, below)
     if (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && ct.bm == 256)) return launch_one<TYPES>(t, ct, s, false, true);
   }

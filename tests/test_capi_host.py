@@ -121,11 +121,17 @@ def test_plan_headline_configs(capi):
 
 
 def test_plan_split_launch_and_offset_limits(capi):
-    # 324 tiles of 256x256 on 256 compute units: whole rounds first, the remaining rows as a second launch
-    p = capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 0, 1)
-    assert (p.tile_m, p.tile_n, p.grid) == (256, 256, 252) and p.tail_rows == 1024 and p.tail_grid > 0
-    assert capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 1, 1).tail_rows == 0      # column-major A: rows are not packed
-    assert capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 0, 1, capi.RUNG_MFMA, 6).tail_rows == 0
+    # 272 tiles of 256x256 on 256 compute units, row-major B (no stream-K): whole rounds first, the remaining rows
+    # as a second launch
+    p = capi.plan(capi.BF16BF16F32, 4352, 4096, 4096, 0, 0)
+    assert (p.tile_m, p.tile_n, p.grid) == (256, 256, 256) and p.tail_rows == 256 and p.tail_grid > 0
+    # column-major A and B: the same cut on the transposed problem, i.e. over columns of the real one
+    p = capi.plan(capi.BF16BF16F32, 4096, 4352, 4096, 1, 1)
+    assert (p.tile_m, p.tile_n, p.grid) == (256, 256, 256) and p.tail_rows == 0 and p.tail_cols == 256 and p.tail_grid > 0
+    # 324 tiles: 68 remain, which the persistent launch carries better than a second launch
+    p = capi.plan(capi.BF16BF16F32, 4608, 4608, 4608, 0, 0)
+    assert p.tail_rows == 0 and p.grid == 256
+    assert capi.plan(capi.BF16BF16F32, 4352, 4096, 4096, 0, 0, capi.RUNG_MFMA, 6).tail_rows == 0
     assert capi.plan(capi.BF16BF16F32, 4096, 4096, 4096, 0, 1).tail_rows == 0      # exactly one round
     # the streaming kernels address rows with 32-bit byte offsets: a K of 20 million goes to the tiled rung
     assert capi.plan(capi.BF16BF16BF16, 64, 64, 20_000_000, 0, 1).rung == capi.RUNG_MFMA
@@ -176,10 +182,11 @@ def test_column_cut_weighs_k(capi):
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (3, 16, 3)
     p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 1, 0)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (8, 128, 128)
-    # row-major A and B: a cut along the columns would put the first launch on the register-staged kernel (a column
-    # range of a row-major B is not a packed matrix); the rows are cut instead, and both launches keep their kernels
+    # row-major A and B: a column range of a row-major B keeps the pitch of the whole matrix, which the ring kernel
+    # takes as a leading dimension while its rows are whole 16-byte pieces (4104 fp16 are); with N = 4100 they are not,
+    # a column cut would put the first launch on the register-staged kernel, and the rows are cut instead
     p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 0)
-    assert p.tail_cols == 0 and p.tail_rows == 256 and (p.tile_m, p.tile_n) == (256, 256)
+    assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (8, 128, 128) and (p.tile_m, p.tile_n) == (256, 256) and p.variant in (5, 6)
     # with a K-contiguous B the sixteen tiles of that seventeenth tile column are cut along K instead (stream-K)
     p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 1)
     assert p.tail_cols == 0 and p.streamk_tiles == 16
