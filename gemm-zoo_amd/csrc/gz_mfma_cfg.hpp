@@ -154,7 +154,8 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       if (direct && rem) shape_cost = (double)full + 0.72 + (frac > 0.5 ? 0.56 * (frac - 0.5) : 0.0);
       // below one round (on eight waves, which such a grid gets): 0.77 up to half a round of tiles, rising to a
       // whole one (bf16 K = 4096, us: 81 tiles 74, 128 75, 144 78, 160 80, 192 88 against 97 for 256)
-      if (direct && full == 0) shape_cost = 0.77 + (frac > 0.5 ? 0.46 * (frac - 0.5) : 0.0);
+      // (the 8-bit floats 0.81: e4m3 M x 4096 x 4096, 16 ... 128 tiles 40.2 - 40.8 us against 51 for 256)
+      if (direct && full == 0) shape_cost = (f8_types ? 0.81 : 0.77) + (frac > 0.5 ? 0.46 * (frac - 0.5) : 0.0);
     }
     // fp32 is bound by its matrix rate at every tile size, so a smaller tile costs what its share of the products
     // costs: 256 x 128 half a round per round of its own, 128 x 128 its tiles over four per compute unit (measured,
@@ -173,14 +174,30 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // rounds of 256 x 256, bf16 K = 4096 - 324 tiles 0.70, 504 0.81, 512 0.80, 576 1.09, 640 1.11, 768 1.19 (the line
     // below said 0.99 for the first three and 1.27 for the others, and 2300^2 x 4096 ran 256 x 256 tiles in 82 us
     // instead of these in 67)
+    // The 8-bit floats' 128 x 128 tiles (their own direct-to-LDS kernel; no ring instance).  Measured in rounds of
+    // 256 x 256 tiles, M x 4096 x 4096 and x 2048, e4m3 - K-contiguous B, one work-group per compute unit at a time:
+    // 64 tiles 0.36 / 0.40, 256 0.43 / 0.45, 384 0.65 / 0.66, 512 0.73 / 0.72, 768 1.05 / 1.00, 1024 1.36 / 1.31;
+    // row-major B, two at a time: 64 0.59 / 0.58, 256 0.63 / 0.61, 512 0.70 / 0.70, 768 1.26 / 1.23, 1024 1.36 / 1.34.
+    bool f8_rowb_fitted = false;
+    if (i == 2 && direct && f8_types) {
+      if (b_cols) {
+        shape_cost = tiles <= num_cus ? 0.36 + 0.07 * (double)tiles / num_cus
+                                      : 0.12 + 0.31 * rounds + 0.035 * (rounds > 4 ? rounds - 4 : 0);
+      } else {
+        const long long full2 = tiles / (2LL * num_cus), rem2 = tiles % (2LL * num_cus);
+        shape_cost = 0.68 * full2 + (rem2 ? 0.58 + 0.12 * (double)rem2 / (2.0 * num_cus) : 0.0) + 0.05 * (full2 > 2 ? full2 - 2 : 0);
+        f8_rowb_fitted = true;
+      }
+    }
     bool fitted128 = false;
     if (i == 2 && !direct && !f32 && tiles <= 3LL * num_cus) {
       shape_cost = tiles <= 2LL * num_cus ? 0.50 + 0.30 * (double)tiles / (2.0 * num_cus)
                                           : 1.06 + 0.13 * (double)(tiles - 2LL * num_cus) / num_cus;
       // Against a grid of 256 x 256 tiles below one round these start and end faster and cost more per slab (512
       // tiles against 128 of 256 x 256, ragged, bf16, us: K = 2048 41.5 / 45.8, K = 4096 75.0 / 74.9 - lines of
-      // 8 + 1.03 per slab and 16.7 + 0.91 per slab); the figures above are those of K = 4096.
-      if (tiles <= 2LL * num_cus) {
+      // 8 + 1.03 per slab and 16.7 + 0.91 per slab); the figures above are those of K = 4096.  (Not with a row-major
+      // B, where the smaller tile's transposing reads take the gain back: K = 2048 47.3 / 44.5.)
+      if (tiles <= 2LL * num_cus && b_cols) {
         const double nslab = (double)K * in_size / MFMA_SLAB_BYTES;
         double kf = (8.0 + 1.03 * nslab) / (16.7 + 0.91 * nslab) / 0.987;
         shape_cost *= kf < 0.88 ? 0.88 : kf > 1.06 ? 1.06 : kf;
@@ -191,7 +208,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     if (f32 && i == 2) shape_cost = 0.10 + 1.15 * (double)tiles / (4.0 * num_cus);
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
     // (the ring kernel takes a row-major B through the transposing reads at no cost to speak of, on either tile)
-    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : ring128_ok ? 1.0 : 1.15) : 1.0;
+    const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : ring128_ok || f8_rowb_fitted ? 1.0 : 1.15) : 1.0;
     // What the register-staged kernel costs over a direct-to-LDS one on the same tile (4096 x 4096 x 4000 against
     // 4096^3, us: bf16 256 x 256 on eight waves 121 / 100, 128 x 128 155 against an estimated 150; int8 73 / 58 and
     // 98 / 87; fp8, four waves, 81 / 52 and 92 / 90).  On 128 x 128 tiles it grows with the rounds beyond four (twice

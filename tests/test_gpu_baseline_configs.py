@@ -181,7 +181,7 @@ def test_ragged_m_n_on_the_hand_scheduled_kernels(G, types, shape, lb):
         assert np.array_equal(got[r], ref[r])
 
 
-@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.F16F16F16])
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.F16F16F16, O.E4M3E4M3F16])
 @pytest.mark.parametrize("shape,lb", [((4352, 4096), O.ROW), ((7168, 7168), O.ROW), ((4352, 4096), O.COL)])
 def test_mostly_empty_last_round_runs_as_two_launches(G, types, shape, lb):
     """272 (or 784) tiles of 256x256 on 256 compute units leave a last round of 16 tiles: the launcher cuts the rows
