@@ -423,7 +423,13 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         return GZ_OK;
       }
       MfmaSplit tsp;
-      if (MfmaCfg ct; mfma_transposed_ring(types, m, n, k, layoutA, layoutB, variant, num_cus, &ct, &tsp)) {
+      // (column-major A and B: a few columns past a multiple of 256 are cut off first, as launch_mfma does)
+      MfmaColSplit ccs;
+      const bool cc_cut = variant == 0 && k > 0 && layoutA == GZ_COL_MAJOR && layoutB == GZ_COL_MAJOR &&
+                          mfma_resolve_colsplit(types, m, n, k, layoutA, layoutB, num_cus, &ccs);
+      const int n_ring = cc_cut ? ccs.cols_main : n;   // columns that the transposed problem covers
+      if (MfmaCfg ct; mfma_transposed_ring(types, m, n_ring, k, layoutA, layoutB, variant, num_cus, &ct, cc_cut ? nullptr : &tsp)) {
+        if (cc_cut) tsp.rows_main = 0;
         // column-major A and B: the ring kernel on the transposed problem (as launch_mfma, aligned operands assumed);
         // the configuration's rows run along N there
         plan->variant = ct.id;
@@ -431,7 +437,7 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         plan->wave_m = ct.bn / ct.waves_m; plan->wave_n = ct.bm / ct.waves_n;
         plan->threads = ct.waves_m * ct.waves_n * 64;
         plan->lds_bytes = mfma_lds_bytes(ct);
-        const int n_first = tsp.rows_main > 0 ? tsp.rows_main : n;   // columns of the first launch
+        const int n_first = tsp.rows_main > 0 ? tsp.rows_main : n_ring;   // columns of the first launch
         plan->grid = (int64_t)ceil_div(n_first, ct.bm) * ceil_div(m, ct.bn);
         if (ct.ring == 1 && mfma_shape_class(ct, es, n_first, m, k, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE)
           plan->grid = mfma_persistent_grid(plan->grid, num_cus);
@@ -440,6 +446,12 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
           plan->tail_tile_m = tsp.tail.bn;
           plan->tail_tile_n = tsp.tail.bm;
           plan->tail_grid = (int64_t)ceil_div(n - tsp.rows_main, tsp.tail.bm) * ceil_div(m, tsp.tail.bn);
+        }
+        if (cc_cut) {   // the cut-off columns: dot products, or tiles of the problem as given
+          plan->tail_cols = n - ccs.cols_main;
+          plan->tail_tile_m = ccs.strip ? 16 : ccs.tail.bm;
+          plan->tail_tile_n = ccs.strip ? plan->tail_cols : ccs.tail.bn;
+          plan->tail_grid = ccs.strip ? ceil_div(m, 16) : (int64_t)ceil_div(m, ccs.tail.bm) * ceil_div(n - ccs.cols_main, ccs.tail.bn);
         }
         if (plan->lds_bytes > lds_per_cu) {
           set_error("mfma variant %d needs %d bytes of LDS, device has %d", ct.id, plan->lds_bytes, lds_per_cu);

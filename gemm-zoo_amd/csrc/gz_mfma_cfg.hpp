@@ -378,6 +378,8 @@ struct MfmaColSplit {
   MfmaCfg main, tail;
   bool strip;         // the cut-off columns run as dot products (mfma_strip_kernel), not as tiles
 };
+inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, int layoutB, int variant, int num_cus,
+                                 MfmaCfg* out, MfmaSplit* split);
 inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, int layoutB, int num_cus, MfmaColSplit* out,
                                   double* estimate = nullptr) {
   out->cols_main = 0;
@@ -385,10 +387,16 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   const int r = N % 256;
   if (N < 512 || r == 0 || r > 64 || M <= 0 || K <= 0) return false;
   MfmaCfg single;
-  const double cost_single = mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, &single);
+  double cost_single = mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, &single);
   const int cols_main = N - r;
   MfmaCfg main_cfg, tail_cfg;
   double cost_main = mfma_choose(types, M, cols_main, K, layoutA, layoutB, num_cus, &main_cfg);
+  // (column-major A and B: what the ring kernel on the transposed problem costs, where it takes the whole problem
+  // and where it takes the first launch)
+  if (MfmaCfg t; mfma_transposed_ring(types, M, N, K, layoutA, layoutB, 0, num_cus, &t, nullptr))
+    cost_single = mfma_choose(types, N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, &t);
+  if (MfmaCfg t; mfma_transposed_ring(types, M, cols_main, K, layoutA, layoutB, 0, num_cus, &t, nullptr))
+    cost_main = mfma_choose(types, cols_main, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, &t);
   // the first launch keeps the ring kernel on a 256 x 256 tile where the layouts allow it and the rows of a
   // row-major B, which keep the pitch of the whole matrix, are whole 16-byte pieces
   const int cls = mfma_shape_class(main_cfg, mfma_in_size(types), M, cols_main, K, layoutA, layoutB);

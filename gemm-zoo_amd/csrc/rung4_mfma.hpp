@@ -1402,13 +1402,18 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
   const int num_cus = device_compute_units();
   g.store_hint = mfma_store_hint(TYPES, g.M, g.N, g.K, (int)sizeof(typename Traits<TYPES>::out_t), num_cus);
   // Column-major A and B: the transposed problem on the ring kernel - one launch, or where the launcher would cut
-  // the rows of the transposed problem (a mostly empty last round) two, over column ranges of the real C and D
-  MfmaSplit tsp;
-  if (MfmaCfg ct; mfma_transposed_ring(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, variant, num_cus, &ct, &tsp)) {
-    GemmArgs<TYPES> t = g;
-    t.A = g.B; t.B = g.A;
-    t.M = g.N; t.N = g.M;
-    t.lda = g.ldb; t.ldb = g.lda;
+  // the rows of the transposed problem (a mostly empty last round) two, over column ranges of the real C and D.
+  // Returns -1 where that kernel does not take the problem.
+  auto run_transposed = [&](const GemmArgs<TYPES>& gm, bool allow_split) -> int {
+    MfmaSplit tsp;
+    MfmaCfg ct;
+    if (!mfma_transposed_ring(TYPES, gm.M, gm.N, gm.K, gm.layoutA, gm.layoutB, variant, num_cus, &ct, allow_split ? &tsp : nullptr))
+      return -1;
+    if (!allow_split) tsp.rows_main = 0;
+    GemmArgs<TYPES> t = gm;
+    t.A = gm.B; t.B = gm.A;
+    t.M = gm.N; t.N = gm.M;
+    t.lda = gm.ldb; t.ldb = gm.lda;
     t.layoutA = GZ_ROW_MAJOR; t.layoutB = GZ_ROW_MAJOR;
     auto cls_of = [&](const GemmArgs<TYPES>& a, const MfmaCfg& c) {
       return mfma_launch_class(c, (int)sizeof(typename Traits<TYPES>::in_t), (int)sizeof(typename Traits<TYPES>::out_t), a.M, a.N,
@@ -1432,6 +1437,24 @@ template <int TYPES> int launch_mfma(const GemmArgs<TYPES>& args, int variant, h
     const int cls = cls_of(t, ct);
     // (unaligned operands, or rows of D that are not: the kernels of the problem as given, below)
     if (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && ct.bm == 256)) return launch_one<TYPES>(t, ct, s, false, true);
+    return -1;
+  };
+  // (a few columns past a multiple of 256 are cut off first, as for the other layouts: the transposed problem would
+  // carry them as a whole row of tiles - bf16 4096 x 4104 x 4096 170 us in one launch)
+  MfmaColSplit ccs;
+  if (variant == 0 && g.K > 0 && g.layoutA == GZ_COL_MAJOR && g.layoutB == GZ_COL_MAJOR &&
+      mfma_resolve_colsplit(TYPES, g.M, g.N, g.K, g.layoutA, g.layoutB, num_cus, &ccs)) {
+    GemmArgs<TYPES> left = g, right = g;
+    left.N = ccs.cols_main;
+    right.N = g.N - ccs.cols_main;
+    right.B = g.B + (size_t)ccs.cols_main * (size_t)g.ldb;
+    if (g.C) right.C = g.C + ccs.cols_main;
+    right.D = g.D + ccs.cols_main;
+    const int st = run_transposed(left, false);
+    if (st > 0) return st;
+    if (st == GZ_OK) return ccs.strip ? launch_strip<TYPES>(right, s) : launch_one<TYPES>(right, ccs.tail, s, true);
+  } else if (const int st = run_transposed(g, true); st >= 0) {
+    return st;
   }
   if ((variant == 0 || variant == MFMA_VARIANT_STREAMK_W4 || variant == MFMA_VARIANT_STREAMK_W8) && g.K > 0) {
     StreamKPlan skp;

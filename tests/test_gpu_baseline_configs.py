@@ -268,6 +268,24 @@ def test_columns_past_a_multiple_of_256_run_as_a_second_launch(G, types, shape):
     assert split_seen or (types in O.FP8_TYPES and n % 256 > 8)
 
 
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32, O.E4M3E4M3F16])
+@pytest.mark.parametrize("shape", [(4096, 4104, 512), (2048, 8200, 256), (4000, 4160, 384)])
+def test_column_major_pair_cuts_columns_before_the_transposed_launch(G, types, shape):
+    """Column-major A and B with a few columns past a multiple of 256 and whole K slabs: the columns up to the
+    multiple run as the transposed problem on the ring kernel, the rest as dot products or small tiles of the problem
+    as given.  First and last rows, every column (the seam included), alpha and beta at work, against the oracle."""
+    m, n, k = shape
+    p = G.capi.plan(types, m, n, k, O.COL, O.COL)
+    assert p.variant in (5, 6) and (p.tile_m, p.tile_n) == (256, 256) and p.tail_cols == n % 256 and p.tail_rows == 0
+    assert p.grid == -(-m // 256) * (n // 256) and p.tail_grid > 0
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+    a, b, c = O.make_inputs(types, m, n, k, kind=kind, seed=11)
+    got = G.run_gemm(types, a, b, c, m, n, k, O.COL, O.COL, 2, -1, -1)
+    for rows in ((0, 24), (m // 2 - 8, m // 2 + 8), (m - 24, m)):
+        ref = O.gemm(types, a, b, c, m, n, k, O.COL, O.COL, 2, -1, rows=rows)
+        assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, shape, rows)
+
+
 def test_ragged_baseline_shape_is_split_by_columns(G):
     p = G.capi.plan(O.F16F16F16, 4095, 4097, 1023, O.ROW, O.ROW)
     assert (p.tile_m, p.tile_n, p.grid, p.tail_cols, p.tail_tile_m, p.tail_grid) == (256, 256, 256, 1, 16, 256)
