@@ -34,11 +34,12 @@ static const MfmaCfg kMfmaCfgs[] = {
     {9, 256, 256, 2, 2, 2, false},   // variant 5 with one work-group per tile (for comparisons with the persistent launch)
     {10, 256, 256, 2, 4, 2, false},  // variant 6, the same
     {11, 128, 128, 2, 2, 2, false},  // tile of variant 3 on the ring kernel, two work-groups per compute unit
+    {12, 64, 64, 2, 2, 0, false},    // four waves of 32x32: grids that 128x128 tiles leave mostly empty
 };
 constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
 // positions in the table
 enum { MFMA_CFG_256_W4 = 0, MFMA_CFG_256_W8 = 1, MFMA_CFG_128 = 2, MFMA_CFG_256x128 = 3, MFMA_CFG_RING_W4 = 4,
-       MFMA_CFG_RING_W8 = 5, MFMA_CFG_RING_128 = 10 };
+       MFMA_CFG_RING_W8 = 5, MFMA_CFG_RING_128 = 10, MFMA_CFG_64 = 11 };
 enum { MFMA_VARIANT_RING_W4 = 5, MFMA_VARIANT_RING_W8 = 6, MFMA_VARIANT_STREAMK_W4 = 7, MFMA_VARIANT_STREAMK_W8 = 8 };
 
 // the most any kernel of the configuration asks for: the ring kernel keeps five buffers of half a slab each
@@ -121,13 +122,38 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   // (fp32: the 256 x 256 tile on four waves with a row-major A)
   const bool ring_ok = types == GZ_F32F32F32 ? a_rows : a_direct;
   const bool ring128_ok = ring_ok && !f8_types && types != GZ_F32F32F32;
-  const int cand[3] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,
-                       ring128_ok ? MFMA_CFG_RING_128 : MFMA_CFG_128};
+  const int cand[4] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,
+                       ring128_ok ? MFMA_CFG_RING_128 : MFMA_CFG_128, MFMA_CFG_64};
   double best = 0;
   int pick = cand[0];
-  for (int i = 0; i < 3; i++) {
+  for (int i = 0; i < 4; i++) {
     const MfmaCfg& c = kMfmaCfgs[cand[i]];
     const long long tiles = (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+    if (i == 3) {
+      // 64 x 64 tiles on the register-staged kernel, several work-groups per compute unit: for grids that larger
+      // tiles leave mostly empty.  No 8-bit instance.
+      double cost64 = -1.0;
+      if (types == GZ_F32F32F32) {
+        // A 128 x 128 tile is 55 us of fp32 products per 1024 of K on one compute unit, whatever the grid.  A
+        // sixteenth of a round of 256 x 256 per tile at 0.75 of the larger tiles' rate (us, 64 x 64 / 128 x 128 tiles,
+        // cubes, row/row: 256 8.1 / 21.0, 512 13.7 / 37.3, 1024 25.4 / 70.2, 1536 86.0 / 103.4, 2048 149.5 / 136.7).
+        const double share = (double)tiles / (16.0 * num_cus);
+        cost64 = (0.05 + 1.35 * (share > 1.0 / 16 ? share : 1.0 / 16)) * 2.2;
+      } else if (in_size == 2 && tiles * 5 <= (b_cols ? 8LL : 6LL) * num_cus) {
+        // 16-bit types, up to 1.6 tiles per compute unit (1.2 with a row-major B: 1280^2 x 2048 22.1 / 20.5, with a
+        // K-contiguous B 18.5 / 20.0): a tile costs 1.3 + 0.49 us per slab against the
+        // 16 + 1.45 of a round of 256 x 256 (us, 64 x 64 / 128 x 128 ring, bf16 -> f32 cubes, row/col: 256 4.7 / 6.3,
+        // 512 5.2 / 7.6, 768 7.5 / 10.6, 1024 9.1 / 12.4, 1280 12.5 / 14.5, 1536 18.8 / 16.6; row/row 1024
+        // 10.5 / 12.8, 1280 14.8 / 14.9; fp16 the same).
+        const double nslab = (double)K * in_size / MFMA_SLAB_BYTES, t = (double)tiles / num_cus;
+        cost64 = (1.3 + 0.49 * nslab) / (16.0 + 1.45 * nslab) * (t <= 1.0 ? 0.8 + 0.2 * t : 1.0 + 0.45 * (t - 1.0));
+      }
+      if (cost64 >= 0 && cost64 < best) {
+        best = cost64;
+        pick = cand[i];
+      }
+      continue;
+    }
     const long long rounds = (tiles + num_cus - 1) / num_cus;
     // whole tiles: every candidate has a direct-to-LDS kernel; ragged M or N: the 256x256 ones only
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
@@ -205,7 +231,8 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       fitted128 = true;
     }
     if (f32 && i == 1) shape_cost = 0.52 * rounds;
-    if (f32 && i == 2) shape_cost = 0.10 + 1.15 * (double)tiles / (4.0 * num_cus);
+    // (a grid of fewer 128 x 128 tiles than compute units still takes a whole tile's time)
+    if (f32 && i == 2) shape_cost = 0.10 + 1.15 * (tiles > num_cus ? (double)tiles / (4.0 * num_cus) : 0.25);
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
     // (the ring kernel takes a row-major B through the transposing reads at no cost to speak of, on either tile)
     const double rowb = (direct && !b_cols) ? (i == 0 ? 1.0 : i == 1 ? 1.12 : ring128_ok || f8_rowb_fitted ? 1.0 : 1.15) : 1.0;
@@ -294,6 +321,8 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
   if (variant < 0 || variant > kNumMfmaCfgs) return false;
   if (variant > 0) {
     *out = kMfmaCfgs[variant - 1];
+    // (the 64 x 64 tile's transposing stores need two 16-byte pieces per lane and row block: no 8-bit instance)
+    if (out->bm == 64 && mfma_in_size(types) == 1) *out = kMfmaCfgs[MFMA_CFG_128];
     return true;
   }
   (void)mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, out);
@@ -419,7 +448,10 @@ inline bool mfma_resolve_colsplit(int types, int M, int N, int K, int layoutA, i
   // of 108).
   const double k_units = (double)K * mfma_in_size(types) / 2048.0, m_units = (double)M / 4096.0;
   const double round_us = 16.0 + 1.45 * ((double)K * mfma_in_size(types) / 128.0);
-  const double strip_us = 3.0 + m_units * k_units * (4.0 + 1.8 * r), tiles_us = 5.0 + 11.5 * m_units * k_units;
+  // (a column-major A is read by the dot products in pieces of rows, a line of memory per k: 2.5 x - col/col
+  // 4096 x 4099 x 4096 took 200 us with the strip against 172 in one launch)
+  const double strip_us = (3.0 + m_units * k_units * (4.0 + 1.8 * r)) * (layoutA == GZ_ROW_MAJOR ? 1.0 : 2.5),
+               tiles_us = 5.0 + 11.5 * m_units * k_units;
   out->strip = r <= MFMA_STRIP_MAX_COLS && strip_us <= tiles_us;
   const double cost_tail = (out->strip ? strip_us : tiles_us) / round_us;
   if (cost_main + cost_tail > 0.97 * cost_single) return false;
@@ -575,9 +607,10 @@ inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, in
     auto whole = [&](const MfmaCfg& c, int rows) {
       return c.ring != 0 && !c.stream_k && mfma_shape_class(c, in_size, rows, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE;
     };
+    // (the remaining rows on the ring kernel's small tile where the estimate took a tile that kernel does not have)
     if (split && types != GZ_F32F32F32 && types != GZ_E4M3E4M3F16 && types != GZ_E5M2E5M2F16 &&
         mfma_resolve_split(types, N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, &sp) && whole(sp.main, sp.rows_main) &&
-        whole(sp.tail, N - sp.rows_main)) {
+        whole(sp.tail.ring ? sp.tail : (sp.tail = kMfmaCfgs[MFMA_CFG_RING_128]), N - sp.rows_main)) {
       *split = sp;
       *out = sp.main;
     }

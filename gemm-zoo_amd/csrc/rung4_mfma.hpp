@@ -260,7 +260,9 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       });
     } else if constexpr (RAGGED) {
       // eight rows at a time: their LDS reads first, then the stores, so that a row does not wait for the one before
-      constexpr int RG = 8, NC = COLS / 64;
+      // (a sub-tile 32 columns wide: the upper half of the lanes has no column)
+      constexpr int RG = 8, NC = (COLS + 63) / 64;
+      const bool has_col = COLS % 64 == 0 || lane < COLS % 64;   // in the last group of 64 columns
       for (int r0 = 0; r0 < 32; r0 += RG) {
         const int mg = row0 + 32 * I + r0;
         if (mg >= M) break;
@@ -269,7 +271,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
           constexpr int R = decltype(r_c)::value;
           static_for<NC>([&](auto c_c) {
             constexpr int C = decltype(c_c)::value;
-            __builtin_memcpy(&v[R][C], region + (r0 + R) * PITCH_E + (C * 64 + lane) * 4, 4);
+            v[R][C] = 0;
+            if (C < NC - 1 || has_col) __builtin_memcpy(&v[R][C], region + (r0 + R) * PITCH_E + (C * 64 + lane) * 4, 4);
           });
         });
         static_for<RG>([&](auto r_c) {
@@ -278,7 +281,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
           static_for<NC>([&](auto c_c) {
             constexpr int C = decltype(c_c)::value;
             const int nn = col0 + C * 64 + lane;
-            if (m < M && nn < N) g.D[(size_t)m * LDD + nn] = epilogue<TYPES>(v[R][C], g.alpha, g.beta, g.C + (size_t)m * LDC + nn);
+            if (m < M && nn < N && (C < NC - 1 || has_col))
+              g.D[(size_t)m * LDD + nn] = epilogue<TYPES>(v[R][C], g.alpha, g.beta, g.C + (size_t)m * LDC + nn);
           });
         });
       }
@@ -1359,6 +1363,9 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
     case 9: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s, transposed);
     case 10: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s, transposed);
     case 11: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 2, s, transposed);
+    case 12:   // (8-bit elements have no such instance: mfma_resolve hands out the 128 x 128 tile for them)
+      if constexpr (sizeof(in_t) >= 2) return launch_cfg<TYPES, 64, 64, 2, 2>(g, edge, 0, s);
+      break;
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);

@@ -150,7 +150,8 @@ def test_plan_streamk(capi):
     """Host-only planning of the stream-K decomposition (nothing is launched)."""
     MF = capi.RUNG_MFMA
     # 272 tiles on 256 compute units: a whole round, and 16 tiles whose slabs are dealt to further work-groups
-    p = capi.plan(capi.BF16BF16F32, 4352, 4096, 4096, 0, 1)
+    # (from a long K on: at K = 4096 the remaining rows as a launch of 64 x 64 tiles cost the same or less)
+    p = capi.plan(capi.BF16BF16F32, 4352, 4096, 8192, 0, 1)
     assert p.variant in (7, 8) and p.streamk_tiles == 16 and p.streamk_blocks % 8 == 0 and p.streamk_blocks > 16
     assert p.grid == 256 + p.streamk_blocks and p.tail_rows == 0 and p.tail_cols == 0
     assert p.workspace_bytes == (p.streamk_blocks + 16 - 1) * 256 * 256 * 4
@@ -178,17 +179,30 @@ def test_column_cut_weighs_k(capi):
     """A few columns past a multiple of 256: dot products while K is short, 128 x 128 tiles once K makes them cheaper."""
     p = capi.plan(capi.F16F16F16, 4096, 4097, 1024, 0, 1)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (1, 16, 1)
-    p = capi.plan(capi.F16F16F16, 4096, 4099, 4096, 0, 1)
+    # (row-major A and B with rows of B that are not whole 16-byte pieces: no ring kernel, no row cut that pays)
+    p = capi.plan(capi.F16F16F16, 4096, 4099, 4096, 0, 0)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (3, 16, 3)
+    # a K-contiguous B: the last rows as a launch of 64 x 64 tiles beside a first launch of 255 tiles of 256 x 256
+    p = capi.plan(capi.F16F16F16, 4096, 4099, 4096, 0, 1)
+    assert (p.tail_rows, p.tail_cols, p.tail_tile_m, p.tail_tile_n, p.grid) == (256, 0, 64, 64, 255)
+    # a column-major A makes the dot products expensive: tiles from a shorter K on
+    p = capi.plan(capi.F16F16F16, 4096, 4099, 4096, 1, 1)
+    assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (3, 128, 128)
     p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 1, 0)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (8, 128, 128)
     # row-major A and B: a column range of a row-major B keeps the pitch of the whole matrix, which the ring kernel
     # takes as a leading dimension while its rows are whole 16-byte pieces (4104 fp16 are); with N = 4100 they are not,
     # a column cut would put the first launch on the register-staged kernel, and the rows are cut instead
-    p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 0)
+    p = capi.plan(capi.F16F16F16, 2048, 8200, 4096, 0, 0)
     assert (p.tail_cols, p.tail_tile_m, p.tail_tile_n) == (8, 128, 128) and (p.tile_m, p.tile_n) == (256, 256) and p.variant in (5, 6)
-    # with a K-contiguous B the sixteen tiles of that seventeenth tile column are cut along K instead (stream-K)
-    p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 1)
+    # (4096 x 4104: the last 256 rows as a launch of 64 x 64 tiles cost less than the strip of eight columns)
+    p = capi.plan(capi.F16F16F16, 4096, 4104, 4096, 0, 0)
+    assert (p.tail_rows, p.tail_cols, p.tail_tile_m, p.variant) == (256, 0, 64, 6)
+    p = capi.plan(capi.F16F16F16, 4096, 4100, 4096, 0, 0)
+    assert p.tail_cols == 4 and p.variant == 2
+    # with a K-contiguous B and a long K the sixteen tiles of that seventeenth tile column are cut along K instead
+    # (stream-K)
+    p = capi.plan(capi.F16F16F16, 4096, 4104, 8192, 0, 1)
     assert p.tail_cols == 0 and p.streamk_tiles == 16
 
 

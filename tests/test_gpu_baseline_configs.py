@@ -127,16 +127,21 @@ def test_c5_skinny_bf16(G, m):
 
 @pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16])
 @pytest.mark.parametrize("shape,tile,variant", [((4096, 4096, 512), (256, 256), 0), ((2048, 4096, 1024), (128, 128), 0),
-                                                ((2048, 4096, 1024), (256, 128), 4), ((512, 384, 256), (128, 128), 0),
-                                                ((256, 128, 128), (128, 128), 0), ((512, 384, 256), (128, 128), 3)])
+                                                ((2048, 4096, 1024), (256, 128), 4), ((512, 384, 256), (64, 64), 0),
+                                                ((256, 128, 128), (64, 64), 0), ((512, 384, 256), (128, 128), 3),
+                                                ((512, 384, 256), (128, 128), 11), ((256, 128, 128), (128, 128), 11)])
 def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile, variant):
     """Row-major A and B (every driver of the reference).  The first shape gives each compute unit a whole 256x256
     tile (hand-scheduled ring kernel, transposing LDS reads for B), the others take the smaller tiles without
-    predication: 128x128 on the same ring kernel with two work-groups per compute unit (the launcher's choice), 256x128
-    on the register-staged kernel and 128x128 on the compiler-scheduled direct-to-LDS kernel (variants 4 and 3)."""
+    predication: 128x128 on the same ring kernel with two work-groups per compute unit (the launcher's choice, and
+    variant 11 on the small grids), 64x64 on the register-staged kernel where larger tiles would leave most compute
+    units idle (the launcher's choice for 16- and 32-bit elements; int8 stays on 128x128), 256x128 on the
+    register-staged kernel and 128x128 on the compiler-scheduled direct-to-LDS kernel (variants 4 and 3)."""
     m, n, k = shape
     p = G.capi.plan(types, m, n, k, O.ROW, O.ROW, 4 if variant else -1, variant)
     assert p.rung == 4 and m % p.tile_m == 0 and n % p.tile_n == 0          # whole tiles: no predicated kernel
+    if tile == (64, 64) and types == O.S8S8S32:
+        tile = (128, 128)
     assert (p.tile_m, p.tile_n) == tile
     kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT   # exact partial sums in any order
     a, b, ha, hb = device_inputs(G, types, m, n, k, kind, 77)
@@ -194,7 +199,7 @@ def test_mostly_empty_last_round_runs_as_two_launches(G, types, shape, lb):
     assert short.tail_rows == 0, "a short K is one launch"
     assert G.capi.plan(types, 4608, 4608, k, O.ROW, lb).tail_rows == 0, "68 remaining tiles are one launch"
     p = G.capi.plan(types, m, n, k, O.ROW, lb)
-    assert p.rung == 4 and (p.tile_m, p.tile_n) == (256, 256) and 0 < p.tail_rows < m and p.tail_tile_m in (128, 256)
+    assert p.rung == 4 and (p.tile_m, p.tile_n) == (256, 256) and 0 < p.tail_rows < m and p.tail_tile_m in (64, 128, 256)
     main_tiles = (m - p.tail_rows) // 256 * -(-n // 256)   # past one round of the compute units one work-group per CU walks them
     assert (m - p.tail_rows) % 256 == 0 and p.grid == min(main_tiles, G.capi.device_props()[0]) and p.tail_grid > 0
     # an explicit variant is one launch
