@@ -121,7 +121,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   const bool a_direct = a_rows || (!b_cols && !f8_types);
   // (fp32: the 256 x 256 tile on four waves with a row-major A)
   const bool ring_ok = types == GZ_F32F32F32 ? a_rows : a_direct;
-  const bool ring128_ok = ring_ok && !f8_types && types != GZ_F32F32F32;
+  const bool ring128_ok = ring_ok && !f8_types;
   const int cand[4] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,
                        ring128_ok ? MFMA_CFG_RING_128 : MFMA_CFG_128, MFMA_CFG_64};
   double best = 0;
@@ -157,7 +157,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const long long rounds = (tiles + num_cus - 1) / num_cus;
     // whole tiles: every candidate has a direct-to-LDS kernel; ragged M or N: the 256x256 ones only
     const int cls = mfma_shape_class(c, in_size, M, N, K, layoutA, layoutB);
-    const bool direct = (types == GZ_F32F32F32 ? a_rows && i == 0 : a_direct) &&
+    const bool direct = (types == GZ_F32F32F32 ? a_rows && (i == 0 || i == 2) : a_direct) &&
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     // (128 x 128 beyond four rounds: each further round costs a little more, 6144^2 x 6144 = 9 rounds measured
     // 478 us against 457 for three rounds of 256 x 256)
@@ -192,7 +192,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // 27.8, 2560 39.0, 3072 74.7 against rounds of 34, 44, 55, 65, 76); the register-staged kernel of the same tile,
     // which the launcher keeps for a K-contiguous B while every work-group has a compute unit to itself, within 0.04
     // of that.
-    if (i == 2 && direct && ring128_ok) {
+    if (i == 2 && direct && ring128_ok && types != GZ_F32F32F32) {
       const long long full2 = tiles / (2LL * num_cus), rem2 = tiles % (2LL * num_cus);
       shape_cost = 0.66 * full2 + (rem2 ? 0.36 + 0.15 * (double)rem2 / num_cus : 0.0);
     }
@@ -230,7 +230,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       }
       fitted128 = true;
     }
-    if (f32 && i == 1) shape_cost = 0.52 * rounds;
+    // (256 x 128 at 0.55 per round of its own: 2560^3, 200 tiles, 313 us against 286 on 400 tiles of 128 x 128 on the
+    // ring kernel and 568 for a round of 256 x 256)
+    if (f32 && i == 1) shape_cost = 0.55 * rounds;
     // (a grid of fewer 128 x 128 tiles than compute units still takes a whole tile's time)
     if (f32 && i == 2) shape_cost = 0.10 + 1.15 * (tiles > num_cus ? (double)tiles / (4.0 * num_cus) : 0.25);
     // row-major B: the compiler-scheduled kernels of the smaller tiles lose more to the transposing reads
@@ -264,7 +266,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     // 21.1 / 23.1, f16 37.1 / 42.9, bf16 35.7 / 41.3; K = 1024: 9.6 / 9.7, 13.5 / 14.5, 13.1 / 14.1), as for a
     // row-major B at every size (1024 13.8 / 18.6, 2048 27.9 / 39.9; int8 1024^3 9.3 / 10.9).
     const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
-    if (b_cols && types != GZ_BF16BF16F32 && tiles <= num_cus * 5LL / 8) *out = kMfmaCfgs[MFMA_CFG_128];
+    if (b_cols && types != GZ_BF16BF16F32 && types != GZ_F32F32F32 && tiles <= num_cus * 5LL / 8) *out = kMfmaCfgs[MFMA_CFG_128];
   }
   if (pick == MFMA_CFG_RING_W4) {
     // Waves per 256 x 256 tile on the ring kernel.
@@ -621,7 +623,7 @@ inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, in
   // (and their slab schedule wants eight row blocks per wave, which the eight-wave tile laid out the other way round
   // does not have: four waves)
   if ((f8 || types == GZ_F32F32F32) && out->waves_m * out->waves_n == 8) *out = kMfmaCfgs[out->id - 2];
-  if (types == GZ_F32F32F32 && out->bm != 256) return false;
+  if (types == GZ_F32F32F32 && out->bm != 256 && out->id != kMfmaCfgs[MFMA_CFG_RING_128].id) return false;
   const int cls = mfma_shape_class(*out, mfma_in_size(types), N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR);
   return cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && out->bm == 256);
 }

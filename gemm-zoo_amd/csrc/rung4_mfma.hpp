@@ -1071,6 +1071,19 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
       else GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
     }
   }
+  // (and the 128 x 128 tile of the same kernel on whole tiles, two work-groups per compute unit)
+  if constexpr (TYPES == GZ_F32F32F32 && BM == 128 && BN == 128 && WAVES_M == 2 && WAVES_N == 2) {
+    if (transposed) {
+      if (ring && !edge)
+        GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, false, false, false, true>), ring_lds, StreamK{});
+      set_error("mfma rung: no kernel for the transposed problem on this tile");
+      return GZ_ERR_UNSUPPORTED;
+    }
+    if (ring && akc && !edge) {
+      if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});
+      else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false>), ring_lds, StreamK{});
+    }
+  }
   if constexpr (TYPES != GZ_F32F32F32) {
     // `transposed`: g is the transposed problem of a column-major A with a column-major B (see SWAP in
     // rung4_mfma_ring16.hpp), a row-major pair for the ring kernel's operands, with the real C and D

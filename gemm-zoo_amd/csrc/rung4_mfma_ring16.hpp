@@ -183,7 +183,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_PW = BM / 16 / NW, B_PW = BN / 16 / NW;  // 1 KiB copies (8 rows) per wave and group
   constexpr int NCP = A_PW + B_PW;
-  static_assert(!F32 || (BM == 256 && BN == 256 && NW == 4 && A_KC && !STREAMK), "fp32: the 256 x 256 tile on four waves, row-major A");
+  static_assert(!F32 || (NW == 4 && A_KC && !STREAMK), "fp32: four waves, row-major A");
   static_assert((BM == 256 && BN == 256) || (BM == 128 && BN == 128 && NW == 4 && !F8 && !STREAMK),
                 "the 256 x 256 tile, or the 128 x 128 tile on four waves for int8 and the 16-bit types");
   static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile rows must divide over the waves");
