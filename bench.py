@@ -269,6 +269,14 @@ def main() -> int:
         t32 = flops / (r32["kernel_ms_mean"] * 1e-3) / 1e12
         extras["f32_4096_row_row"] = {"tflops": round(t32, 2), "frac_of_f32_peak": round(t32 / PEAK_TFLOPS["f32"], 4),
                                       "kernel_ms_mean": round(r32["kernel_ms_mean"], 5)}
+        # the small cubes of the same drivers (nvidia/bench/bench_tiling.cu and its siblings start at 128^3): 64 x 64
+        # tiles, so that a grid of a few dozen output tiles still reaches every compute unit
+        small = {}
+        for sz in (512, 1024, 2048):
+            rsm = timed(capi.F32F32F32, sz, sz, sz, capi.ROW_MAJOR, capi.ROW_MAJOR, 100, 100)
+            small[str(sz)] = {"tflops": round(2.0 * sz ** 3 / (rsm["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                              "kernel_us_mean": round(rsm["kernel_ms_mean"] * 1e3, 2)}
+        extras["f32_small_cubes_row_row"] = small
         # the two remaining configurations of the baseline: int8 1024^3 (row-major A and B) and the ragged fp16
         # problem 4095 x 4097 x 1023 (row-major A and B, predicated edge tiles, unaligned rows)
         rs1 = timed(capi.S8S8S32, 1024, 1024, 1024, capi.ROW_MAJOR, capi.ROW_MAJOR, 100, 100)
@@ -297,6 +305,14 @@ def main() -> int:
                 extras[name] = {"tflops": round(2.0 * sz ** 3 / (rl["kernel_ms_mean"] * 1e-3) / 1e12, 2),
                                 "kernel_ms_mean": round(rl["kernel_ms_mean"], 5)}
                 lt.close()
+            small = {}
+            for sz in (512, 1024, 2048):
+                lt = functors.HipblasLtGemm(capi.F32F32F32, sz, sz, sz, capi.ROW_MAJOR, capi.ROW_MAJOR)
+                rl = timed(capi.F32F32F32, sz, sz, sz, capi.ROW_MAJOR, capi.ROW_MAJOR, 100, 100, vendor=lt)
+                small[str(sz)] = {"tflops": round(2.0 * sz ** 3 / (rl["kernel_ms_mean"] * 1e-3) / 1e12, 2),
+                                  "kernel_us_mean": round(rl["kernel_ms_mean"] * 1e3, 2)}
+                lt.close()
+            extras["hipblaslt_f32_small_cubes_row_row"] = small
         except Exception as e:  # the comparator is optional: report why it is absent, never fail the bench for it
             extras["hipblaslt"] = {"unavailable": str(e)[:200]}
         sk = {}
