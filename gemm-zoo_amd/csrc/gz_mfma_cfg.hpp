@@ -382,9 +382,7 @@ inline bool mfma_resolve_split(int types, int M, int N, int K, int layoutA, int 
   double cost_main = mfma_choose(types, rows_main, N, K, layoutA, layoutB, num_cus, &main_cfg);
   if (main_cfg.bm != 256 || main_cfg.bn != 256) return false;
   // only where the first launch runs a direct-to-LDS kernel, whose speed the estimate knows well
-  if (types == GZ_F32F32F32 ||
-      mfma_shape_class(main_cfg, mfma_in_size(types), rows_main, N, K, layoutA, layoutB) == MFMA_SHAPE_GENERAL)
-    return false;
+  if (mfma_shape_class(main_cfg, mfma_in_size(types), rows_main, N, K, layoutA, layoutB) == MFMA_SHAPE_GENERAL) return false;
   const double cost_tail = mfma_choose(types, M - rows_main, N, K, layoutA, layoutB, num_cus, &tail_cfg);
   if (cost_main + cost_tail > 0.97 * cost_single) return false;
   if (estimate) *estimate = cost_main + cost_tail;
@@ -610,7 +608,7 @@ inline bool mfma_transposed_ring(int types, int M, int N, int K, int layoutA, in
       return c.ring != 0 && !c.stream_k && mfma_shape_class(c, in_size, rows, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE;
     };
     // (the remaining rows on the ring kernel's small tile where the estimate took a tile that kernel does not have)
-    if (split && types != GZ_F32F32F32 && types != GZ_E4M3E4M3F16 && types != GZ_E5M2E5M2F16 &&
+    if (split && types != GZ_E4M3E4M3F16 && types != GZ_E5M2E5M2F16 &&
         mfma_resolve_split(types, N, M, K, GZ_ROW_MAJOR, GZ_ROW_MAJOR, num_cus, &sp) && whole(sp.main, sp.rows_main) &&
         whole(sp.tail.ring ? sp.tail : (sp.tail = kMfmaCfgs[MFMA_CFG_RING_128]), N - sp.rows_main)) {
       *split = sp;
