@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel means of the counters of one or more `rocprofv3 --pmc ... --output-format csv` runs.
 
-    python3 gemm-zoo_amd/bench/pmc_table.py gpurun_out/pmc_a gpurun_out/pmc_b [--skip fill,elementwise]
+    python3 gemm-zoo_amd/bench/pmc_table.py out/pmc_a out/pmc_b [--skip fill,elementwise]
 
 Every directory is searched for *counter_collection.csv; one line per (kernel, counter): mean, minimum and maximum
 over the dispatches of that kernel, and their number.  With --levels the dispatches of a kernel are also grouped by

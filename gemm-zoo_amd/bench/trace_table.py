@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel durations of a `rocprofv3 --kernel-trace --output-format csv` run, leg by leg.
 
-    python3 gemm-zoo_amd/bench/trace_table.py gpurun_out/prof_stats [--min-run 100] [--window 200:800]
+    python3 gemm-zoo_amd/bench/trace_table.py out/prof_stats [--min-run 100] [--window 200:800]
 
 A process like bench.py launches the same kernel for several workloads one after the other (beta = 0, then
 alpha = beta = 1).  The dispatches of a kernel are therefore cut into RUNS - maximal sequences in start order that no
