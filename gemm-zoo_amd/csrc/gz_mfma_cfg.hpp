@@ -479,7 +479,7 @@ inline int mfma_resolve_cut(int types, int M, int N, int K, int layoutA, int lay
 // contiguous runs; a run covers the end of one tile or that and the start of the next, leaves its sums in a slot of
 // a workspace, and a second small launch adds each tile's pieces in a fixed order and writes D (the reference has the
 // same tail: its persistent grid of min(#SM, tiles) work-groups, nvidia/kernel_functors/bf16_mma_gemm.cuh:42-48).
-// Only on the kernel with the 16x16 instructions: row-major A, column-major B, whole K slabs, 16-byte aligned rows.
+// Only on the kernel with the 16x16 instructions: row-major A, either layout of B, whole K slabs, 16-byte aligned rows.
 struct StreamKPlan {
   int dp_tiles, sk_tiles, blocks, q, rem;   // see struct StreamK of the kernel
   int slots;                                // workspace slots of 256 x 256 accumulators
@@ -492,7 +492,7 @@ inline bool mfma_plan_streamk(int types, int M, int N, int K, int layoutA, int l
                               const MfmaCfg* forced_cfg, StreamKPlan* out) {
   if (num_cus <= 0) num_cus = 256;
   const int in_size = mfma_in_size(types);
-  if (!(types == GZ_S8S8S32 || in_size == 2) || layoutA != GZ_ROW_MAJOR || layoutB != GZ_COL_MAJOR) return false;
+  if (!(types == GZ_S8S8S32 || in_size == 2) || layoutA != GZ_ROW_MAJOR) return false;
   MfmaCfg cfg;
   double single_rounds = mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, &cfg);
   if (forced) cfg = kMfmaCfgs[forced_cfg->waves_n == 4 ? MFMA_CFG_RING_W8 : MFMA_CFG_RING_W4];

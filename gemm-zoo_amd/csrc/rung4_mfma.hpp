@@ -1401,15 +1401,18 @@ static int launch_streamk(const GemmArgs<TYPES>& g, const StreamKPlan& p, bool r
     const int tiles_m = ceil_div(g.M, 256), tiles_n = ceil_div(g.N, 256);
     const dim3 grid((unsigned)(p.dp_tiles + p.blocks)), block(2 * WAVES_N * 64);
     const size_t rlds = 5u * (size_t)(256 + 256) * 64;
-    if (ragged) {
-      auto kern = mfma_ring16_kernel<TYPES, 256, 256, 2, WAVES_N, true, true>;
-      GZ_SET_LDS_LIMIT(kern, rlds);
-      hipLaunchKernelGGL(kern, grid, block, rlds, s, g, tiles_m, tiles_n, sk);
-    } else {
-      auto kern = mfma_ring16_kernel<TYPES, 256, 256, 2, WAVES_N, false, true>;
-      GZ_SET_LDS_LIMIT(kern, rlds);
-      hipLaunchKernelGGL(kern, grid, block, rlds, s, g, tiles_m, tiles_n, sk);
-    }
+#define GZ_LAUNCH_SK(RAGGED_, BKC_)                                                    \
+  do {                                                                                 \
+    auto kern = mfma_ring16_kernel<TYPES, 256, 256, 2, WAVES_N, RAGGED_, true, BKC_>;  \
+    GZ_SET_LDS_LIMIT(kern, rlds);                                                      \
+    hipLaunchKernelGGL(kern, grid, block, rlds, s, g, tiles_m, tiles_n, sk);           \
+  } while (0)
+    const bool bkc = g.layoutB == GZ_COL_MAJOR;
+    if (ragged && bkc) GZ_LAUNCH_SK(true, true);
+    else if (ragged) GZ_LAUNCH_SK(true, false);
+    else if (bkc) GZ_LAUNCH_SK(false, true);
+    else GZ_LAUNCH_SK(false, false);
+#undef GZ_LAUNCH_SK
     GZ_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL((streamk_fixup_kernel<TYPES>), dim3((unsigned)p.sk_tiles * 64), dim3(256), 0, s, g, tiles_m, tiles_n, sk);
     GZ_HIP_TRY(hipGetLastError());

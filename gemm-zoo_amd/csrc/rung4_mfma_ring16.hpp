@@ -175,7 +175,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int EPV = 16 / ES;
   constexpr int HK = 64 / ES;         // K rows of a row-major B per copy group: one K step
   constexpr bool F8 = is_fp8(TYPES);
-  static_assert(B_KC || !STREAMK, "stream-K with a column-major B only");
+  static_assert(!STREAMK || (A_KC && !SWAP), "stream-K with a row-major A (either layout of B)");
   static_assert(!SWAP || !B_KC, "the transposed problem of two column-major operands has a row-major second operand");
   static_assert(!(F8 && STREAMK), "stream-K for int8 and the 16-bit types");
   static_assert(A_KC || (!B_KC && !SWAP && !STREAMK && !F8), "a column-major A with a row-major B, int8 and the 16-bit types");

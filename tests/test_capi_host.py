@@ -165,7 +165,9 @@ def test_plan_streamk(capi):
     p = capi.plan(capi.S8S8S32, 5120, 5120, 5120, 0, 1, MF, 7)
     assert p.variant == 7 and p.streamk_tiles == 144 and p.streamk_blocks == 256 and p.threads == 256
     assert capi.plan(capi.F16F16F16, 5120, 5120, 5120, 0, 1, MF, 8).threads == 512
-    for args in [(capi.BF16BF16F32, 5120, 5120, 5120, 0, 0), (capi.BF16BF16F32, 5120, 5120, 5120, 1, 1),
+    # (a row-major B as well: its copies carry whole K rows, and a run starts at a K row of its own)
+    assert capi.plan(capi.BF16BF16F32, 5120, 5120, 5120, 0, 0, MF, 7).streamk_tiles == 144
+    for args in [(capi.BF16BF16F32, 5120, 5120, 5120, 1, 0), (capi.BF16BF16F32, 5120, 5120, 5120, 1, 1),
                  (capi.F32F32F32, 5120, 5120, 5120, 0, 1), (capi.E4M3E4M3F16, 5120, 5120, 5120, 0, 1),
                  (capi.BF16BF16F32, 5120, 5120, 5100, 0, 1), (capi.BF16BF16F32, 256, 256, 64, 0, 1)]:
         p = capi.plan(*args, MF, 7)
