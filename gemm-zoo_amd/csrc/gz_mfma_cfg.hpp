@@ -114,12 +114,12 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
   if (num_cus <= 0) num_cus = 256;
   const int in_size = mfma_in_size(types);
   const bool a_rows = layoutA == GZ_ROW_MAJOR, b_cols = layoutB == GZ_COL_MAJOR;
-  // candidates: 256x256 (on the ring kernel where the types and the layout of A allow it), 256x128, 128x128
+  // candidates: 256x256 and 128x128 (on the ring kernel where the types and the layout of A allow it), 256x128, 64x64
   // (a column-major A beside a row-major B goes through the transposing reads like B, not for the 8-bit floats; beside
   // a column-major B the launcher runs the transposed problem where it can, see mfma_transposed_ring)
   const bool f8_types = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
   const bool a_direct = a_rows || (!b_cols && !f8_types);
-  // (fp32: the 256 x 256 tile on four waves with a row-major A)
+  // (fp32: four waves with a row-major A)
   const bool ring_ok = types == GZ_F32F32F32 ? a_rows : a_direct;
   const bool ring128_ok = ring_ok && !f8_types;
   const int cand[4] = {ring_ok ? MFMA_CFG_RING_W4 : MFMA_CFG_256_W4, MFMA_CFG_256x128,

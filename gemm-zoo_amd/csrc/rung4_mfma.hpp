@@ -15,11 +15,13 @@
 //                      Slabs are staged global -> registers -> LDS ([row][k], pitch 144 B: the 16-byte pad
 //                      makes the fragment reads of 16 consecutive rows hit 16 distinct 4-bank groups);
 //                      operands whose contiguous dimension is not K (row-major B, column-major A) are
-//                      transposed in registers on the way in.
+//                      transposed in registers on the way in.  Tiles 256x256, 256x128, 128x128 and, for
+//                      grids that those leave mostly empty, 64x64 (16- and 32-bit elements).
 //   mfma_dtl_kernel    compiler-scheduled fast path for whole tiles with 16-byte aligned rows: slabs go
 //                      global -> LDS directly (global_load_lds_dwordx4), unpadded swizzled rows.
-//   mfma_ring16_kernel (rung4_mfma_ring16.hpp) the hand-scheduled 256 x 256 kernel with the 16x16 matrix
-//                      instructions and a ring of five LDS buffers: what the launcher runs on big problems.
+//   mfma_ring16_kernel (rung4_mfma_ring16.hpp) the hand-scheduled kernel with the 16x16 matrix instructions
+//                      and a ring of five LDS buffers, on 256 x 256 and 128 x 128 tiles: what the launcher
+//                      runs wherever operands are aligned and K is whole slabs.
 //
 // Stands in for nvidia/kernels/sm_80/{bf16,fp16}_mma_gemm.cuh and
 // intel/kernels/xe_gemm_*_m8k16.hpp (same operation, new design).
@@ -1044,8 +1046,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
   // The direct-to-LDS kernels: row-major A, whole K slabs, 16-byte aligned rows (the shape class says so), whole
   // tiles or, on the hand-scheduled 256 x 256 kernel, any M and N (rows clamped).  ring: 0 the compiler-scheduled
   // kernels, 1 the hand-scheduled ring kernel with one work-group per compute unit walking the tiles of a grid of
-  // more than one round, 2 the same kernel with one work-group per tile.  fp32 runs the register-staged kernel only:
-  // its MFMAs are 8x longer per byte.
+  // more than one round, 2 the same kernel with one work-group per tile.
   constexpr bool TILE_256 = BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4);
   const size_t ring_lds = 5u * (size_t)(BM + BN) * 64;
   const size_t dtl_lds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
