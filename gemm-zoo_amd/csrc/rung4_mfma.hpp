@@ -573,6 +573,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
 
   StagerA sa;
   StagerB sb;
+  // The 64 x 64 tile has so few matrix instructions per slab (sixteen per wave) that a slab asked for one iteration
+  // ahead has not arrived when its turn comes, and a work-group that is alone on its compute unit waits for it in
+  // every iteration: it keeps TWO slabs in flight, in two sets of registers that take turns.
+  constexpr bool DEEP = BM == 64 && BN == 64 && !is_fp8(TYPES);
+  constexpr int LEAD = DEEP ? 3 : 2;   // a slab is asked for LEAD iterations before it is multiplied
+  StagerA sa2;
+  StagerB sb2;
 
   acc_v acc[FM][FN];
 #pragma unroll
@@ -644,34 +651,59 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   using LoadPredicated = std::integral_constant<int, 0>;
   using LoadInside = std::integral_constant<int, 1>;
   using LoadNothing = std::integral_constant<int, 2>;
-  auto load_slab = [&](auto mode_c, int k0) __attribute__((always_inline)) {
+  auto load_slab = [&](auto mode_c, int k0, StagerA& xa, StagerB& xb) __attribute__((always_inline)) {
     constexpr int MODE = decltype(mode_c)::value;
     if constexpr (MODE == 1) {
-      sa.load_inside(g.A, g.M, g.K, m0, k0, tid, (size_t)g.lda);
-      sb.load_inside(g.B, g.N, g.K, n0, k0, tid, (size_t)g.ldb);
+      xa.load_inside(g.A, g.M, g.K, m0, k0, tid, (size_t)g.lda);
+      xb.load_inside(g.B, g.N, g.K, n0, k0, tid, (size_t)g.ldb);
     } else if constexpr (MODE == 0) {
-      sa.load(g.A, g.M, g.K, m0, k0, tid, (size_t)g.lda);
-      sb.load(g.B, g.N, g.K, n0, k0, tid, (size_t)g.ldb);
+      xa.load(g.A, g.M, g.K, m0, k0, tid, (size_t)g.lda);
+      xb.load(g.B, g.N, g.K, n0, k0, tid, (size_t)g.ldb);
     }
   };
-  auto load_slab_checked = [&](int slab) __attribute__((always_inline)) {
+  auto load_slab_checked = [&](int slab, StagerA& xa, StagerB& xb) __attribute__((always_inline)) {
     if constexpr (PEEL) {
       if (slab < full_slabs) {
-        load_slab(LoadInside{}, slab * BK);
+        load_slab(LoadInside{}, slab * BK, xa, xb);
         return;
       }
     }
-    load_slab(LoadPredicated{}, slab * BK);
+    load_slab(LoadPredicated{}, slab * BK, xa, xb);
   };
-  // Prologue: slab 0 into LDS, slab 1 parked in registers, fragments of (slab 0, step 0) requested.
-  load_slab_checked(0);
+  // Prologue: slab 0 into LDS, slab 1 parked in registers (DEEP: and slab 2 in the second set), fragments of
+  // (slab 0, step 0) requested.
+  load_slab_checked(0, sa, sb);
   sa.store(lds, tid);
   sb.store(lds + A_BYTES, tid);
-  if (ktiles > 1) load_slab_checked(1);
+  if (ktiles > 1) load_slab_checked(1, sa, sb);
+  if constexpr (DEEP) {
+    if (ktiles > 2) load_slab_checked(2, sa2, sb2);
+  }
   __syncthreads();
   read_frags(0, lds, 0);
-  // iterations whose loads (slab kt + 2) are inside: the first kt_inside of them
-  const int kt_inside = PEEL ? max(0, min(ktiles, full_slabs - 2)) : 0;
+  // iterations whose loads (slab kt + LEAD) are inside: the first kt_inside of them
+  const int kt_inside = PEEL ? max(0, min(ktiles, full_slabs - LEAD)) : 0;
+  // iteration kt parks slab kt + 1 from the register set of its parity (the only set unless DEEP) and refills it
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  auto run_iters = [&](auto&& iter, auto mode_c, int& kt, int end) __attribute__((always_inline)) {
+    if constexpr (!DEEP) {
+      for (; kt < end; kt++) iter(mode_c, Set0{}, kt);
+    } else {
+      if ((kt & 1) && kt < end) {
+        iter(mode_c, Set1{}, kt);
+        kt++;
+      }
+      for (; kt + 1 < end; kt += 2) {
+        iter(mode_c, Set0{}, kt);
+        iter(mode_c, Set1{}, kt + 1);
+      }
+      if (kt < end) {
+        iter(mode_c, Set0{}, kt);
+        kt++;
+      }
+    }
+  };
 
   // Steady state per slab (KSTEPS = 4 MFMA steps), one barrier per slab:
   //   step 0 : request step 1's fragments; the parked registers (slab kt+1) go to the other LDS buffer, which every
@@ -696,14 +728,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
           acc[i][j] = mfma_f8_pair<TYPES>(bf[2 * pair][j], bf[2 * pair + 1][j], af[2 * pair][i], af[2 * pair + 1][i], acc[i][j]);
     };
     read_frags(1, lds, 1);
-    auto slab_iter = [&](auto mode_c, int kt) __attribute__((always_inline)) {
+    auto slab_iter = [&](auto mode_c, auto /*set_c*/, int kt) __attribute__((always_inline)) {
       const char* cur = lds + (kt & 1) * STAGE_BYTES;
       char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
       read_frags(2, cur, 2);
       read_frags(3, cur, 3);
       sa.store(nxt, tid);
       sb.store(nxt + A_BYTES, tid);
-      load_slab(mode_c, (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK);
+      load_slab(mode_c, (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK, sa, sb);
       mma2(0);
       mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, FM * FN>();
       __builtin_amdgcn_sched_barrier(0);
@@ -715,20 +747,20 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       __builtin_amdgcn_sched_barrier(0);
     };
     int kt = 0;
-    if constexpr (PEEL)
-      for (; kt < kt_inside; kt++) slab_iter(LoadInside{}, kt);
-    for (; kt < (PEEL ? ktiles - 2 : ktiles); kt++) slab_iter(LoadPredicated{}, kt);
-    if constexpr (PEEL)
-      for (; kt < ktiles; kt++) slab_iter(LoadNothing{}, kt);
+    if constexpr (PEEL) run_iters(slab_iter, LoadInside{}, kt, kt_inside);
+    run_iters(slab_iter, LoadPredicated{}, kt, PEEL ? ktiles - 2 : ktiles);
+    if constexpr (PEEL) run_iters(slab_iter, LoadNothing{}, kt, ktiles);
   } else {
-    auto slab_iter = [&](auto mode_c, int kt) __attribute__((always_inline)) {
+    auto slab_iter = [&](auto mode_c, auto set_c, int kt) __attribute__((always_inline)) {
       const char* cur = lds + (kt & 1) * STAGE_BYTES;
       char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+      StagerA& xa = [&]() -> StagerA& { if constexpr (decltype(set_c)::value) return sa2; else return sa; }();
+      StagerB& xb = [&]() -> StagerB& { if constexpr (decltype(set_c)::value) return sb2; else return sb; }();
 
       read_frags(1, cur, 1);
-      sa.store(nxt, tid);
-      sb.store(nxt + A_BYTES, tid);
-      load_slab(mode_c, (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK);
+      xa.store(nxt, tid);
+      xb.store(nxt + A_BYTES, tid);
+      load_slab(mode_c, (EDGE || kt + LEAD < ktiles ? kt + LEAD : ktiles - 1) * BK, xa, xb);
       mma(0);
       mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, MFMAS_PER_STEP>();
       __builtin_amdgcn_sched_barrier(0);
@@ -747,11 +779,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
       __builtin_amdgcn_sched_barrier(0);
     };
     int kt = 0;
-    if constexpr (PEEL)
-      for (; kt < kt_inside; kt++) slab_iter(LoadInside{}, kt);
-    for (; kt < (PEEL ? ktiles - 2 : ktiles); kt++) slab_iter(LoadPredicated{}, kt);
-    if constexpr (PEEL)
-      for (; kt < ktiles; kt++) slab_iter(LoadNothing{}, kt);
+    if constexpr (PEEL) run_iters(slab_iter, LoadInside{}, kt, kt_inside);
+    run_iters(slab_iter, LoadPredicated{}, kt, PEEL ? ktiles - LEAD : ktiles);
+    if constexpr (PEEL) run_iters(slab_iter, LoadNothing{}, kt, ktiles);
   }
 
   static_assert(NT / 64 * epilogue_region_bytes<FN>() <= 2 * STAGE_BYTES, "the epilogue reuses the operand buffers");
