@@ -258,16 +258,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     }
   }
   *out = kMfmaCfgs[pick];
-  if (pick == MFMA_CFG_RING_128) {
-    // A K-contiguous B on a grid that leaves a good third of the compute units idle: the register-staged kernel,
-    // whose plain loads get as much out of a lone work-group's path to the L2 and which starts a little faster (us,
-    // ring / register-staged, K = 4096: int8 1024^2 19.2 / 18.6, 1536^2 19.7 / 18.9; f16 33.2 / 32.5, 33.9 / 33.2;
-    // bf16 -> f32 33.4 / 34.9, 33.8 / 35.3).  With every compute unit busy the ring (2048^2, 256 tiles: int8
-    // 21.1 / 23.1, f16 37.1 / 42.9, bf16 35.7 / 41.3; K = 1024: 9.6 / 9.7, 13.5 / 14.5, 13.1 / 14.1), as for a
-    // row-major B at every size (1024 13.8 / 18.6, 2048 27.9 / 39.9; int8 1024^3 9.3 / 10.9).
-    const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
-    if (b_cols && types != GZ_BF16BF16F32 && types != GZ_F32F32F32 && tiles <= num_cus * 5LL / 8) *out = kMfmaCfgs[MFMA_CFG_128];
-  }
+  // (The register-staged kernel of the 128 x 128 tile was kept for a K-contiguous B on grids of up to 5/8 of the compute
+  // units.  Interleaved runs of the two, int8 / fp16 / bf16 -> bf16 squares 512 ... 1536 at K = 1024 ... 8192: the ring
+  // kernel level or 1 - 4 % ahead on all of them but 1536^2 x 8192, 16-bit, 81 against 74 us; the rule is gone.)
   if (pick == MFMA_CFG_RING_W4) {
     // Waves per 256 x 256 tile on the ring kernel.
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
