@@ -139,14 +139,15 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
         // cubes, row/row: 256 8.1 / 21.0, 512 13.7 / 37.3, 1024 25.4 / 70.2, 1536 86.0 / 103.4, 2048 149.5 / 136.7).
         const double share = (double)tiles / (16.0 * num_cus);
         cost64 = (0.05 + 1.35 * (share > 1.0 / 16 ? share : 1.0 / 16)) * 2.2;
-      } else if (in_size == 2 && tiles * 5 <= (b_cols ? 8LL : 6LL) * num_cus) {
-        // 16-bit types, up to 1.6 tiles per compute unit (1.2 with a row-major B: 1280^2 x 2048 22.1 / 20.5, with a
-        // K-contiguous B 18.5 / 20.0): a tile costs 1.3 + 0.49 us per slab against the
+      } else if (in_size == 2 && tiles * 5 <= (b_cols ? 10LL : 6LL) * num_cus) {
+        // 16-bit types, up to two tiles per compute unit (1.2 with a row-major B: 1280^2 x 2048 22.1 / 20.5, with a
+        // K-contiguous B 18.5 / 20.0; 1024 x 2048 x 4096, two per compute unit, 30.1 / 33.5; 1536^2 x 2048, 2.25,
+        // 22.1 / 19.9): a tile costs 1.3 + 0.49 us per slab against the
         // 16 + 1.45 of a round of 256 x 256 (us, 64 x 64 / 128 x 128 ring, bf16 -> f32 cubes, row/col: 256 4.7 / 6.3,
         // 512 5.2 / 7.6, 768 7.5 / 10.6, 1024 9.1 / 12.4, 1280 12.5 / 14.5, 1536 18.8 / 16.6; row/row 1024
         // 10.5 / 12.8, 1280 14.8 / 14.9; fp16 the same).
         const double nslab = (double)K * in_size / MFMA_SLAB_BYTES, t = (double)tiles / num_cus;
-        cost64 = (1.3 + 0.49 * nslab) / (16.0 + 1.45 * nslab) * (t <= 1.0 ? 0.8 + 0.2 * t : 1.0 + 0.45 * (t - 1.0));
+        cost64 = (1.3 + 0.49 * nslab) / (16.0 + 1.45 * nslab) * (t <= 1.0 ? 0.8 + 0.2 * t : 1.0 + 0.35 * (t - 1.0));
       }
       if (cost64 >= 0 && cost64 < best) {
         best = cost64;
