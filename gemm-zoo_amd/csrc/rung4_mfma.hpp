@@ -548,7 +548,6 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_gemm_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
   using in_t = typename T::in_t;
-  using out_t = typename T::out_t;
   using acc_v = typename AccVec<TYPES>::type;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int ES = (int)sizeof(in_t);
@@ -831,7 +830,6 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     mfma_dtl_kernel(GemmArgs<TYPES> g, int tiles_m, int tiles_n) {
   using T = Traits<TYPES>;
   using in_t = typename T::in_t;
-  using out_t = typename T::out_t;
   using acc_v = typename AccVec<TYPES>::type;
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int ES = (int)sizeof(in_t);
