@@ -135,13 +135,11 @@ def test_reference_driver_layout_row_row_direct_kernels(G, types, shape, tile, v
     tile (hand-scheduled ring kernel, transposing LDS reads for B), the others take the smaller tiles without
     predication: 128x128 on the same ring kernel with two work-groups per compute unit (the launcher's choice, and
     variant 11 on the small grids), 64x64 on the register-staged kernel where larger tiles would leave most compute
-    units idle (the launcher's choice for 16- and 32-bit elements; int8 stays on 128x128), 256x128 on the
+    units idle (the launcher's choice; int8 runs that tile on two waves), 256x128 on the
     register-staged kernel and 128x128 on the compiler-scheduled direct-to-LDS kernel (variants 4 and 3)."""
     m, n, k = shape
     p = G.capi.plan(types, m, n, k, O.ROW, O.ROW, 4 if variant else -1, variant)
     assert p.rung == 4 and m % p.tile_m == 0 and n % p.tile_n == 0          # whole tiles: no predicated kernel
-    if tile == (64, 64) and types == O.S8S8S32:
-        tile = (128, 128)
     assert (p.tile_m, p.tile_n) == tile
     kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT   # exact partial sums in any order
     a, b, ha, hb = device_inputs(G, types, m, n, k, kind, 77)
