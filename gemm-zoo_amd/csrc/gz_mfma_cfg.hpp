@@ -37,7 +37,7 @@ static const MfmaCfg kMfmaCfgs[] = {
     {12, 64, 64, 2, 2, 0, false},    // four waves of 32x32: grids that 128x128 tiles leave mostly empty
 };
 constexpr int kNumMfmaCfgs = (int)(sizeof(kMfmaCfgs) / sizeof(kMfmaCfgs[0]));
-// variant 12 for int8: the same tile on two waves of 64x32 (the transposing stores of 8-bit elements need four 16-byte
+// variant 12 for 8-bit elements: the same tile on two waves of 64x32 (the transposing stores of 8-bit elements need four 16-byte
 // pieces per lane and operand, which 128 lanes have on this tile and 256 do not)
 static const MfmaCfg kMfmaCfg64Int8 = {12, 64, 64, 1, 2, 0, false};
 // positions in the table
@@ -134,7 +134,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const long long tiles = (long long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
     if (i == 3) {
       // 64 x 64 tiles on the register-staged kernel, several work-groups per compute unit: for grids that larger
-      // tiles leave mostly empty.  Not for the 8-bit floats; int8 on two waves.
+      // tiles leave mostly empty.  8-bit elements on two waves.
       double cost64 = -1.0;
       if (types == GZ_F32F32F32) {
         // A 128 x 128 tile is 55 us of fp32 products per 1024 of K on one compute unit, whatever the grid.  A
@@ -142,8 +142,8 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
         // cubes, row/row: 256 8.1 / 21.0, 512 13.7 / 37.3, 1024 25.4 / 70.2, 1536 86.0 / 103.4, 2048 149.5 / 136.7).
         const double share = (double)tiles / (16.0 * num_cus);
         cost64 = (0.05 + 1.35 * (share > 1.0 / 16 ? share : 1.0 / 16)) * 2.2;
-      } else if ((in_size == 2 || types == GZ_S8S8S32) && tiles * 5 <= (b_cols ? 10LL : 6LL) * num_cus) {
-        // 16-bit types, up to two tiles per compute unit (1.2 with a row-major B: 1280^2 x 2048 22.1 / 20.5, with a
+      } else if (tiles * 5 <= (b_cols || f8_types ? 10LL : 6LL) * num_cus) {
+        // 8- and 16-bit types, up to two tiles per compute unit (int8 and 16-bit, 1.2 with a row-major B: 1280^2 x 2048 22.1 / 20.5, with a
         // K-contiguous B 18.5 / 20.0; 1024 x 2048 x 4096, two per compute unit, 30.1 / 33.5; 1536^2 x 2048, 2.25,
         // 22.1 / 19.9): a tile costs 1.3 + 0.49 us per slab against the
         // 16 + 1.45 of a round of 256 x 256 (us, 64 x 64 / 128 x 128 ring, bf16 -> f32 cubes, row/col: 256 4.7 / 6.3,
@@ -262,7 +262,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     }
   }
   *out = kMfmaCfgs[pick];
-  if (pick == MFMA_CFG_64 && types == GZ_S8S8S32) *out = kMfmaCfg64Int8;
+  if (pick == MFMA_CFG_64 && in_size == 1) *out = kMfmaCfg64Int8;
   // (The register-staged kernel of the 128 x 128 tile was kept for a K-contiguous B on grids of up to 5/8 of the compute
   // units.  Interleaved runs of the two, int8 / fp16 / bf16 -> bf16 squares 512 ... 1536 at K = 1024 ... 8192: the ring
   // kernel level or 1 - 4 % ahead on all of them but 1536^2 x 8192, 16-bit, 81 against 74 us; the rule is gone.)
@@ -321,8 +321,8 @@ inline bool mfma_resolve(int types, int M, int N, int K, int layoutA, int layout
   if (variant < 0 || variant > kNumMfmaCfgs) return false;
   if (variant > 0) {
     *out = kMfmaCfgs[variant - 1];
-    // (8-bit elements: int8 on two waves, the 8-bit floats have no such instance)
-    if (out->bm == 64 && mfma_in_size(types) == 1) *out = types == GZ_S8S8S32 ? kMfmaCfg64Int8 : kMfmaCfgs[MFMA_CFG_128];
+    // (8-bit elements: on two waves)
+    if (out->bm == 64 && mfma_in_size(types) == 1) *out = kMfmaCfg64Int8;
     return true;
   }
   (void)mfma_choose(types, M, N, K, layoutA, layoutB, num_cus, out);

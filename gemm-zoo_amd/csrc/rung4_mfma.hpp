@@ -1405,10 +1405,9 @@ template <int TYPES> static int launch_one(const GemmArgs<TYPES>& g, const MfmaC
     case 9: return launch_cfg<TYPES, 256, 256, 2, 2>(g, edge, 2, s, transposed);
     case 10: return launch_cfg<TYPES, 256, 256, 2, 4>(g, edge, 2, s, transposed);
     case 11: return launch_cfg<TYPES, 128, 128, 2, 2>(g, edge, 2, s, transposed);
-    case 12:   // (the 8-bit floats have no such instance: mfma_resolve hands out the 128 x 128 tile for them)
+    case 12:   // (8-bit elements on two waves)
       if constexpr (sizeof(in_t) >= 2) return launch_cfg<TYPES, 64, 64, 2, 2>(g, edge, 0, s);
-      else if constexpr (TYPES == GZ_S8S8S32) return launch_cfg<TYPES, 64, 64, 1, 2>(g, edge, 0, s);
-      break;
+      else return launch_cfg<TYPES, 64, 64, 1, 2>(g, edge, 0, s);
     default: break;
   }
   set_error("mfma rung: variant %d not built", cfg.id);
