@@ -143,8 +143,8 @@ typedef struct gz_plan_t {
  * wherever the problem allows it (row-major A, whole K slabs, 16-byte aligned rows; otherwise the kernel of 1 / 2);
  * 7 / 8 the same with the stream-K decomposition; 9 / 10 as 5 / 6 with one work-group per tile instead of one per
  * compute unit; 11 the ring kernel on 128x128 tiles, two work-groups per compute unit (int8, the 16-bit types and
- * fp32; otherwise the kernel of 3); 12 the register-staged kernel on 64x64 tiles (for the 8-bit floats the kernel
- * of 3).                                                                                                       */
+ * fp32; otherwise the kernel of 3); 12 the register-staged kernel on 64x64 tiles (four waves; two for 8-bit
+ * elements).                                                                                                   */
 int gz_gemm_s8s8s32(const int8_t* A, const int8_t* B, const int32_t* C, int32_t* D,
                     int64_t M, int64_t N, int64_t K, int layoutA, int layoutB,
                     int32_t alpha, int32_t beta, int rung, int variant, gz_stream stream);
