@@ -575,7 +575,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
   // The 64 x 64 tile has so few matrix instructions per slab (sixteen per wave) that a slab asked for one iteration
   // ahead has not arrived when its turn comes, and a work-group that is alone on its compute unit waits for it in
   // every iteration: it keeps TWO slabs in flight, in two sets of registers that take turns.
-  constexpr bool DEEP = BM == 64 && BN == 64 && !is_fp8(TYPES);
+  constexpr bool DEEP = BM == 64 && BN == 64;
   constexpr int LEAD = DEEP ? 3 : 2;   // a slab is asked for LEAD iterations before it is multiplied
   StagerA sa2;
   StagerB sb2;
@@ -727,14 +727,16 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
           acc[i][j] = mfma_f8_pair<TYPES>(bf[2 * pair][j], bf[2 * pair + 1][j], af[2 * pair][i], af[2 * pair + 1][i], acc[i][j]);
     };
     read_frags(1, lds, 1);
-    auto slab_iter = [&](auto mode_c, auto /*set_c*/, int kt) __attribute__((always_inline)) {
+    auto slab_iter = [&](auto mode_c, auto set_c, int kt) __attribute__((always_inline)) {
       const char* cur = lds + (kt & 1) * STAGE_BYTES;
       char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+      StagerA& xa = [&]() -> StagerA& { if constexpr (decltype(set_c)::value) return sa2; else return sa; }();
+      StagerB& xb = [&]() -> StagerB& { if constexpr (decltype(set_c)::value) return sb2; else return sb; }();
       read_frags(2, cur, 2);
       read_frags(3, cur, 3);
-      sa.store(nxt, tid);
-      sb.store(nxt + A_BYTES, tid);
-      load_slab(mode_c, (EDGE || kt + 2 < ktiles ? kt + 2 : ktiles - 1) * BK, sa, sb);
+      xa.store(nxt, tid);
+      xb.store(nxt + A_BYTES, tid);
+      load_slab(mode_c, (EDGE || kt + LEAD < ktiles ? kt + LEAD : ktiles - 1) * BK, xa, xb);
       mma2(0);
       mix2_into_mfmas<StagerA::LDS_STORES + StagerB::LDS_STORES, StagerA::VECS + StagerB::VECS, FM * FN>();
       __builtin_amdgcn_sched_barrier(0);
@@ -747,7 +749,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     };
     int kt = 0;
     if constexpr (PEEL) run_iters(slab_iter, LoadInside{}, kt, kt_inside);
-    run_iters(slab_iter, LoadPredicated{}, kt, PEEL ? ktiles - 2 : ktiles);
+    run_iters(slab_iter, LoadPredicated{}, kt, PEEL ? ktiles - LEAD : ktiles);
     if constexpr (PEEL) run_iters(slab_iter, LoadNothing{}, kt, ktiles);
   } else {
     auto slab_iter = [&](auto mode_c, auto set_c, int kt) __attribute__((always_inline)) {
