@@ -439,7 +439,8 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
         plan->lds_bytes = mfma_lds_bytes(ct);
         const int n_first = tsp.rows_main > 0 ? tsp.rows_main : n_ring;   // columns of the first launch
         plan->grid = (int64_t)ceil_div(n_first, ct.bm) * ceil_div(m, ct.bn);
-        if (ct.ring == 1 && mfma_shape_class(ct, es, n_first, m, k, GZ_ROW_MAJOR, GZ_ROW_MAJOR) == MFMA_SHAPE_WHOLE)
+        const int cls_t = mfma_shape_class(ct, es, n_first, m, k, GZ_ROW_MAJOR, GZ_ROW_MAJOR);
+        if (ct.ring == 1 && (cls_t == MFMA_SHAPE_WHOLE || (cls_t == MFMA_SHAPE_RAGGED_MN && ct.bm == 256)))
           plan->grid = mfma_persistent_grid(plan->grid, num_cus);
         if (tsp.rows_main > 0) {   // the remaining columns in a second launch
           plan->tail_cols = n - tsp.rows_main;
@@ -522,10 +523,13 @@ static int plan_impl(int types, int64_t M, int64_t N, int64_t K, int layoutA, in
       plan->threads = c.waves_m * c.waves_n * 64;
       plan->lds_bytes = mfma_lds_bytes(c);
       plan->grid = (int64_t)ceil_div(m_first, c.bm) * ceil_div(n_first, c.bn);
-      // whole tiles on the ring kernel with the 16x16 instructions: one work-group per compute unit walks the tiles
+      // the ring kernel with the 16x16 instructions (whole tiles, or ragged M and N on its 256 x 256 tile): one
+      // work-group per compute unit walks the tiles
+      int cls_g = mfma_shape_class(c, es, m_first, n_first, k, layoutA, layoutB);
+      if (plan->tail_cols && layoutB == GZ_ROW_MAJOR && ((int64_t)n * es) % 16 != 0) cls_g = MFMA_SHAPE_GENERAL;
       if (c.ring == 1 && (layoutA == GZ_ROW_MAJOR || (layoutB == GZ_ROW_MAJOR && !is_fp8(types) && types != GZ_F32F32F32)) &&
           !(types == GZ_F32F32F32 && c.waves_n != 2) &&
-          mfma_shape_class(c, es, m_first, n_first, k, layoutA, layoutB) == MFMA_SHAPE_WHOLE)
+          (cls_g == MFMA_SHAPE_WHOLE || (cls_g == MFMA_SHAPE_RAGGED_MN && c.bm == 256)))
         plan->grid = mfma_persistent_grid(plan->grid, num_cus);
       if (plan->lds_bytes > lds_per_cu) {
         set_error("mfma variant %d needs %d bytes of LDS, device has %d", c.id, plan->lds_bytes, lds_per_cu);

@@ -1076,7 +1076,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
   // The direct-to-LDS kernels: row-major A, whole K slabs, 16-byte aligned rows (the shape class says so), whole
   // tiles or, on the hand-scheduled 256 x 256 kernel, any M and N (rows clamped).  ring: 0 the compiler-scheduled
   // kernels, 1 the hand-scheduled ring kernel with one work-group per compute unit walking the tiles of a grid of
-  // more than one round, 2 the same kernel with one work-group per tile.
+  // more than one round (ragged M and N included), 2 the same kernel with one work-group per tile.
   constexpr bool TILE_256 = BM == 256 && BN == 256 && WAVES_M == 2 && (WAVES_N == 2 || WAVES_N == 4);
   const size_t ring_lds = 5u * (size_t)(BM + BN) * 64;
   const size_t dtl_lds = 2u * (size_t)(BM + BN) * SLAB_BYTES;
@@ -1087,15 +1087,15 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
   if constexpr (TYPES == GZ_F32F32F32 && TILE_256 && WAVES_N == 2) {
     if (transposed) {
       if (ring && shape_class == MFMA_SHAPE_RAGGED_MN)
-        GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, true, false, false, true>), ring_lds, StreamK{});
+        GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, true, false, false, true>), ring_lds, StreamK{});
       if (ring && !edge)
         GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, false, false, false, true>), ring_lds, StreamK{});
       set_error("mfma rung: no kernel for the transposed problem on this tile");
       return GZ_ERR_UNSUPPORTED;
     }
     if (ring && akc && shape_class == MFMA_SHAPE_RAGGED_MN) {
-      if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
-      else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
+      if (bkc) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
+      else GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
     }
     if (ring && akc && !edge) {
       if (bkc) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});
@@ -1122,7 +1122,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
     if (transposed) {
       if constexpr (TILE_256 && !(is_fp8(TYPES) && WAVES_M * WAVES_N == 8)) {
         if (ring && shape_class == MFMA_SHAPE_RAGGED_MN)
-          GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, true, false, false, true>), ring_lds, StreamK{});
+          GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, true, false, false, true>), ring_lds, StreamK{});
         if (ring && !edge)
           GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_N, WAVES_M, false, false, false, true>), ring_lds, StreamK{});
       }
@@ -1137,7 +1137,7 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
     if constexpr (!is_fp8(TYPES)) {
       if constexpr (TILE_256) {
         if (ring && !akc && !bkc && shape_class == MFMA_SHAPE_RAGGED_MN)
-          GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false, false, false>), ring_lds, StreamK{});
+          GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false, false, false>), ring_lds, StreamK{});
         if (ring && !akc && !bkc && !edge)
           GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, false, false, false, false, false>), ring_lds, StreamK{});
       }
@@ -1148,8 +1148,8 @@ static int launch_cfg(const GemmArgs<TYPES>& g, int shape_class, int ring, hipSt
     }
     if constexpr (TILE_256) {
       if (ring && akc && shape_class == MFMA_SHAPE_RAGGED_MN) {
-        if (bkc) GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
-        else GZ_LAUNCH_DIRECT(GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
+        if (bkc) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true>), ring_lds, StreamK{});
+        else GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N, true, false, false>), ring_lds, StreamK{});
       }
       if (ring && akc && !edge) {
         if (bkc) GZ_LAUNCH_DIRECT_ON(pgrid, GZ_KERN(mfma_ring16_kernel<TYPES, BM, BN, WAVES_M, WAVES_N>), ring_lds, StreamK{});

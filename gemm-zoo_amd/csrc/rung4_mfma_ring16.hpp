@@ -211,11 +211,11 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
       it_end = streamk_first_slab(sk, sk_block + 1);
     }
   }
-  // A launch of fewer work-groups than tiles (whole tiles, no stream-K) is a persistent one: work-group b takes
+  // A launch of fewer work-groups than tiles (no stream-K) is a persistent one: work-group b takes
   // tiles b, b + gridDim.x, ... in the order the hardware would have dealt them, and asks for the first slab (copy
   // groups 0 and 1) of its next tile before it stores the current one, so that it arrives during the epilogue
   // instead of after a new work-group's start.
-  constexpr bool PERSISTENT = !STREAMK && !RAGGED;
+  constexpr bool PERSISTENT = !STREAMK;
   int bid = (int)blockIdx.x;
   bool prefetched = false;   // groups 0 and 1 of this pass's tile are already on their way
   for (;;) {
@@ -262,51 +262,53 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
   constexpr int KRC_A = 1024 / (BM * ES), LPR_A = 64 / KRC_A;
   static_assert(A_KC || (KRC_A * BM * ES == 1024 && NW * A_PW * KRC_A == HK), "whole K rows per copy, a K step per group");
   uint32_t voff_a[A_KC ? 2 : 1][A_PW], voff_b[B_KC ? 2 : 1][B_PW];
+  const size_t a_group_step = A_KC ? 0 : (size_t)HK * LDA, b_group_step = B_KC ? 0 : (size_t)HK * LDB;
+  // (the offsets of the tile whose first row and column are m_first, n_first: they differ between tiles only where
+  // RAGGED clamps rows or columns)
+  auto set_copy_offsets = [&](int m_first, int n_first) {
 #pragma unroll
-  for (int par = 0; par < 2; par++) {
-    if constexpr (A_KC) {
+    for (int par = 0; par < 2; par++) {
+      if constexpr (A_KC) {
+#pragma unroll
+        for (int t = 0; t < A_PW; t++) {
+          // RAGGED: rows past the end are fetched from the last row (an output depends on its own row of A and column
+          // of B only, and those past the end are not stored)
+          int r = 16 * (wave * A_PW + t) + 8 * par + ci;
+          if constexpr (RAGGED) r = min(m_first + r, g.M - 1) - m_first;
+          voff_a[par][t] = (uint32_t)((size_t)r * LDA + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+        }
+      }
+      if constexpr (B_KC) {
+#pragma unroll
+        for (int t = 0; t < B_PW; t++) {
+          int r = 16 * (wave * B_PW + t) + 8 * par + ci;
+          if constexpr (RAGGED) r = min(n_first + r, N - 1) - n_first;
+          voff_b[par][t] = (uint32_t)((size_t)r * LDB + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
+        }
+      }
+    }
+    if constexpr (!A_KC) {
+      const int last_piece = (g.M - m_first) / EPV - 1;   // RAGGED: M is a multiple of EPV on this path, m_first < M
 #pragma unroll
       for (int t = 0; t < A_PW; t++) {
-        // RAGGED: rows past the end are fetched from the last row (an output depends on its own row of A and column
-        // of B only, and those past the end are not stored)
-        int r = 16 * (wave * A_PW + t) + 8 * par + ci;
-        if constexpr (RAGGED) r = min(m0 + r, g.M - 1) - m0;
-        voff_a[par][t] = (uint32_t)((size_t)r * LDA + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
+        const int kr = (wave * A_PW + t) * KRC_A + lane / LPR_A;   // K row within the group
+        int piece = (lane % LPR_A) ^ ring16_row_swizzle<ES, BM * ES>(kr);
+        if constexpr (RAGGED) piece = min(piece, last_piece);      // rows past the end: the last piece (not stored)
+        voff_a[0][t] = (uint32_t)((size_t)kr * LDA + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
       }
     }
-    if constexpr (B_KC) {
+    if constexpr (!B_KC) {
+      const int last_piece = (N - n_first) / EPV - 1;   // RAGGED: N is a multiple of EPV on this path, n_first < N
 #pragma unroll
       for (int t = 0; t < B_PW; t++) {
-        int r = 16 * (wave * B_PW + t) + 8 * par + ci;
-        if constexpr (RAGGED) r = min(n0 + r, N - 1) - n0;
-        voff_b[par][t] = (uint32_t)((size_t)r * LDB + (size_t)((cs ^ ci ^ par) * 16)) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
+        const int kr = (wave * B_PW + t) * KRC + lane / LPR;   // K row within the group
+        int piece = (lane % LPR) ^ ring16_row_swizzle<ES, BN * ES>(kr);
+        if constexpr (RAGGED) piece = min(piece, last_piece);  // columns past the end: the last piece (not stored)
+        voff_b[0][t] = (uint32_t)((size_t)kr * LDB + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
       }
     }
-  }
-  size_t a_group_step = 0;
-  if constexpr (!A_KC) {
-    const int last_piece = (g.M - m0) / EPV - 1;   // RAGGED: M is a multiple of EPV on this path, m0 < M
-#pragma unroll
-    for (int t = 0; t < A_PW; t++) {
-      const int kr = (wave * A_PW + t) * KRC_A + lane / LPR_A;   // K row within the group
-      int piece = (lane % LPR_A) ^ ring16_row_swizzle<ES, BM * ES>(kr);
-      if constexpr (RAGGED) piece = min(piece, last_piece);      // rows past the end: the last piece (not stored)
-      voff_a[0][t] = (uint32_t)((size_t)kr * LDA + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - A_PW / 2) * 1024);
-    }
-    a_group_step = (size_t)HK * LDA;
-  }
-  size_t b_group_step = 0;
-  if constexpr (!B_KC) {
-    const int last_piece = (N - n0) / EPV - 1;   // RAGGED: N is a multiple of EPV on this path, n0 < N
-#pragma unroll
-    for (int t = 0; t < B_PW; t++) {
-      const int kr = (wave * B_PW + t) * KRC + lane / LPR;   // K row within the group
-      int piece = (lane % LPR) ^ ring16_row_swizzle<ES, BN * ES>(kr);
-      if constexpr (RAGGED) piece = min(piece, last_piece);  // columns past the end: the last piece (not stored)
-      voff_b[0][t] = (uint32_t)((size_t)kr * LDB + (size_t)(piece * EPV) * ES) + COPY_BIAS - (uint32_t)((t - B_PW / 2) * 1024);
-    }
-    b_group_step = (size_t)HK * LDB;
-  }
+  };
+  set_copy_offsets(m0, n0);
   // scalar bases of a tile: its first row of A (first column of a K-contiguous B) at the first K byte of this run; a
   // row-major B's first K row of the run at the tile's first column
   auto a_base_of = [&](int m_first) -> const char* {
@@ -715,6 +717,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, (BM == 128 && BN == 128
       tile_of_block(next_bid, tiles_m, tiles_n, tm2, tn2);
       const char* const a_next = a_base_of(tm2 * BM);
       const char* const b_next = b_base_of(tn2 * BN);
+      if constexpr (RAGGED) set_copy_offsets(tm2 * BM, tn2 * BN);   // this tile asks for nothing more
       // into buffers 0 and 1, which the epilogue does not use
       issue_group(std::integral_constant<int, 0>{}, a_next, b_next);
       issue_group(std::integral_constant<int, 1>{}, a_next, b_next);

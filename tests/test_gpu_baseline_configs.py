@@ -242,6 +242,32 @@ def test_more_tiles_than_compute_units_on_the_ring_kernel(G, types, variant, sha
     assert np.array_equal(got, one)
 
 
+@pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.F16F16F16, O.E4M3E4M3F16, O.F32F32F32])
+@pytest.mark.parametrize("variant", [5, 6])
+@pytest.mark.parametrize("shape,lb", [((4360, 4096, 3), O.COL), ((8200, 4080, 1), O.ROW), ((4100, 6128, 6), O.COL),
+                                      ((4112, 4336, 2), O.ROW)])
+def test_more_ragged_tiles_than_compute_units_on_the_ring_kernel(G, types, variant, shape, lb):
+    """288, 528, 408 and 289 tiles of 256x256 with a last row and / or column of tiles that reaches past the matrix:
+    the persistent launch of the kernel's ragged instance.  A work-group's next tile may be one whose rows or columns
+    are clamped while its current one is not (and the other way round), so the first copies of the next tile, asked
+    for before the current one is stored, must use the next tile's offsets.  First and last rows, rows of second
+    tiles and the ragged last rows against the oracle; everything against one work-group per tile (variants 9, 10)."""
+    m, n, slabs = shape
+    k = slabs * 128 // np.dtype(O.IN_DTYPE[types]).itemsize
+    kind = O.FILL_INT8_UNIFORM if types == O.S8S8S32 else O.FILL_SMALL_INT
+    ha, hb, hc = O.make_inputs(types, m, n, k, kind=kind, seed=81)
+    p = G.capi.plan(types, m, n, k, O.ROW, lb, 4, variant)
+    print("case", types, variant, shape, lb, p.variant, p.grid, flush=True)
+    # (fp32 has the four-wave instance only: variant 6 runs the register-staged kernel, a work-group per tile)
+    assert p.grid == (-(-m // 256) * -(-n // 256) if types == O.F32F32F32 and variant == 6 else 256)
+    got = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, variant)
+    for rows in ((0, 4), (1020, 1028), (m // 2 - 2, m // 2 + 2), (m // 256 * 256 - 4, m // 256 * 256 + 4), (m - 4, m)):
+        ref = O.gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, rows=rows)
+        assert np.array_equal(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]), (types, variant, shape, lb, rows)
+    one = G.run_gemm(types, ha, hb, hc, m, n, k, O.ROW, lb, 2, 1, 4, variant + 4)
+    assert np.array_equal(got, one)
+
+
 @pytest.mark.parametrize("types", [O.S8S8S32, O.BF16BF16F32, O.BF16BF16BF16, O.F16F16F16, O.F32F32F32, O.E4M3E4M3F16])
 @pytest.mark.parametrize("shape", [(4096, 4097, 72), (2048, 8200, 130), (4095, 4160, 255), (4094, 4099, 1023)])
 def test_columns_past_a_multiple_of_256_run_as_a_second_launch(G, types, shape):
