@@ -271,9 +271,6 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
     const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
     const bool f8 = types == GZ_E4M3E4M3F16 || types == GZ_E5M2E5M2F16;
     bool eight = false;
-    const double nslab_all = (double)K * in_size / MFMA_SLAB_BYTES;
-    const bool ragged = M % 256 != 0 || N % 256 != 0;
-    const bool ragged_eight = ragged && !(b_cols && tiles >= 3LL * num_cus && nslab_all >= (f8 ? 64 : 96));
     if (types == GZ_F32F32F32) {
       eight = false;   // one instance: four waves
     } else if (f8) {
@@ -281,9 +278,7 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // four beyond.  e4m3, us, four / eight waves, row/row: 4096^3 56.2 / 53.3, 5120^3 122.8 / 115.7, 6144^3
       // 221.5 / 213.0, 4096^2 x 8192 99.6 / 99.0, 8192^3 404.9 / 419.4; row/col 4096^3 53.8 / 50.9, 8192^3
       // 386.5 / 401.4.  (A row-major B: eight waves at every size, see below.)
-      // Ragged M or N: eight but for a long K (the four-wave instance that skips rows and columns past the end pays
-      // for it in its epilogue: e4m3 row/col 8000 x 8192 x 2048 177.3 / 148.7, 8000 x 8000 x 8192 392.6 / 396.6).
-      eight = ragged_eight || !(tiles >= 4LL * num_cus && b_cols);
+      eight = !(tiles >= 4LL * num_cus && b_cols);
     } else {
       // int8 and the 16-bit types: an estimate of the launch on four and on eight waves, in us per round of tiles,
       // a fixed part (first copies, epilogue) and a part per K slab.  Eight waves (two per SIMD, 128 x 64 per wave)
@@ -314,13 +309,11 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // Below one round: eight.  With half the compute units idle the busy ones are not held by power, the slopes are
       // the same and eight waves' fixed part is 8 us lower (about 140 tiles, us, four / eight waves, K = 2048 and 4096:
       // row/col 54.3 / 46.0, 86.7 / 78.2; row/row 55.3 / 46.0, 89.3 / 77.6; whole tiles, 3072^2: 79.1 / 76.6, 80.5 / 73.7).
-      // Ragged M or N: eight (ragged_eight).  The four-wave instance that skips rows and columns past the end pays for it in its
-      // epilogue (us, four / eight waves, row/col: bf16 -> f32 4095 x 4096 x 1024 40.1 / 33.0, 4000 x 4096 x 4096
-      // 102.6 / 101.7, 2000 x 8192 x 4096 102.2 / 104.6; fp16 44.9 / 35.5, 109.9 / 106.6, 8000 x 8192 x 2048
-      // 267.8 / 241.0; bf16 -> bf16 row/row 8000 x 8192 x 2048 265.7 / 235.8).
-      // Four waves keep their lower cost per slab: past three rounds of a long K they are ahead again (8000 x 8000
-      // x 8192 row/col: bf16 -> f32 739 / 761, int8 401 / 410).
-      eight = ragged_eight || !a_rows || under_a_round || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
+      // (Ragged M and N follow the same rule: us, four / eight waves, row/col then row/row - bf16 -> f32 4095 x 4096 x
+      // 1024 34.1 / 37.2, 34.8 / 35.6; 8000 x 8192 x 2048 218.6 / 240.9, 222.6 / 242.0; fp16 4095 x 4096 x 1024
+      // 34.3 / 33.8, 35.1 / 32.4; 8000 x 8192 x 2048 219.5 / 230.7, 231.6 / 226.6; int8 8000 x 8000 x 8192 379 / 414,
+      // 402 / 420.)
+      eight = !a_rows || under_a_round || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
     }
     if (eight) *out = kMfmaCfgs[MFMA_CFG_RING_W8];
   }

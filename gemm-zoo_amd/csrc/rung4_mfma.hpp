@@ -148,10 +148,14 @@ __device__ __forceinline__ void store_accumulators(const GemmArgs<TYPES>& g, Acc
 // 16 s + c: acc[i][4 g + s][e] = D(row0 + 16 i + lane % 16, col0 + 64 g + 16 (lane / 16) + 4 e + s) - what a kernel
 // ends up with that feeds the matrix instruction four consecutive columns of a row-major B per lane.  A lane's values
 // of the four blocks of a group are then four consecutive columns again.
-template <int TYPES, int FM, int FN, bool RAGGED = false, int BLK = 32, bool TRANSPOSED = false, bool BY4 = false, class Acc,
-          int AM, int AN>
-__device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g, Acc (&acc)[AM][AN], int row0, int col0,
-                                                       int lane, char* region) {
+// UC: whether C is read - 2: decided here (beta != 0), 0 / 1: known to the caller.  The ragged kernels call it with a
+// constant: their stores sit under each lane's own condition, and where loads of C may be pending when such a region is
+// entered the compiler waits for ALL memory operations there (loads and stores return in no fixed order with respect to
+// each other), i.e. for the previous store, 64 times per wave on the four-wave 256 x 256 tile (7 us per launch).
+// Without loads of C nothing is waited for; with them, they are waited for once per block, before its first store.
+template <int UC, int TYPES, int FM, int FN, bool RAGGED, int BLK, bool TRANSPOSED, bool BY4, class Acc, int AM, int AN>
+__device__ __forceinline__ void store_accumulators_lds_impl(const GemmArgs<TYPES>& g, Acc (&acc)[AM][AN], int row0, int col0,
+                                                            int lane, char* region) {
   static_assert(TRANSPOSED ? (BLK == 16 && AN == FM * 2 && AM == FN * 2)
                            : (AM == FM * (32 / BLK) && AN == FN * (32 / BLK)), "accumulator blocks of BLK x BLK");
   constexpr int NJ = TRANSPOSED ? AM : AN;   // 16-column blocks of a row
@@ -165,7 +169,8 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
   constexpr int LPR = COLS / W, RPI = 64 / LPR, NI = 32 / RPI;   // lanes per row, rows per instruction, instructions
   const int M = g.M, N = g.N;
   const size_t LDC = (size_t)g.ldc, LDD = (size_t)g.ldd;   // elements between the rows of C and of D
-  const bool use_c = g.beta != 0;
+  const bool use_c = UC == 2 ? g.beta != 0 : UC == 1;
+  const typename Traits<TYPES>::scalar_t beta_e = UC == 0 ? (typename Traits<TYPES>::scalar_t)0 : g.beta;   // (UC == 0: beta is 0)
   static_assert(!BY4 || (BLK == 16 && !TRANSPOSED && AN % 4 == 0), "groups of four 16-column blocks");
   char* wr = BLK == 32 ? region + (lane & 31) * PITCH_E + (lane >> 5) * 16
                        : region + (lane & 15) * PITCH_E + (lane >> 4) * (BY4 ? 64 : 16);
@@ -186,18 +191,22 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
       constexpr int T = decltype(t_c)::value;
 #pragma unroll
       for (int e = 0; e < W; e++) cv[T][e] = 0;
-      const int m = row0 + 32 * I + T * RPI + lane / LPR;
-      if (use_c && vec && (!RAGGED || (m < M && n < N))) {
+      // RAGGED: a lane past the last row or column reads the last row / the first columns instead (never stored).
+      // The load itself is unconditional for the wave: under a lane's own condition every load ends in a merge that
+      // waits for it, one load at a time.
+      const int m = RAGGED ? min(row0 + 32 * I + T * RPI + lane / LPR, M - 1) : row0 + 32 * I + T * RPI + lane / LPR;
+      const int nc = RAGGED ? (n < N ? n : 0) : n;
+      if (use_c && vec) {
         if (g.store_hint & 2) {   // non-temporal: see mfma_store_hint
           if constexpr (WB == 16) {
-            const u32x4_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.C + (size_t)m * LDC + n));
+            const u32x4_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(g.C + (size_t)m * LDC + nc));
             __builtin_memcpy(cv[T], &w, 16);
           } else {
-            const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(g.C + (size_t)m * LDC + n));
+            const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(g.C + (size_t)m * LDC + nc));
             __builtin_memcpy(cv[T], &w, 8);
           }
         } else {
-          __builtin_memcpy(cv[T], g.C + (size_t)m * LDC + n, sizeof(cv[T]));
+          __builtin_memcpy(cv[T], g.C + (size_t)m * LDC + nc, sizeof(cv[T]));
         }
       }
     });
@@ -232,10 +241,30 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     if (vec) {
+      // (RAGGED: all of the block's LDS reads first - behind a lane's own condition each would be waited for on its
+      // own, 64 times per wave on the four-wave 256 x 256 tile: 7 us per launch)
+      acc_t vs[RAGGED ? NI : 1][W];
+      if constexpr (RAGGED) {
+        static_for<NI>([&](auto t_c) {
+          constexpr int T = decltype(t_c)::value;
+          __builtin_memcpy(vs[T], rd + T * RPI * PITCH_E, W * 4);
+        });
+        if constexpr (UC == 1) {   // the block's values of C have arrived before the first region of a store is entered
+          static_for<NI>([&](auto t_c) {
+            constexpr int T = decltype(t_c)::value;
+            uint32_t w[WB / 4];
+            __builtin_memcpy(w, cv[T], WB);
+#pragma unroll
+            for (int x = 0; x < WB / 4; x++) asm volatile("" : "+v"(w[x]));
+            __builtin_memcpy(cv[T], w, WB);
+          });
+        }
+      }
       static_for<NI>([&](auto t_c) {
         constexpr int T = decltype(t_c)::value;
         acc_t v[W];
-        __builtin_memcpy(v, rd + T * RPI * PITCH_E, W * 4);
+        if constexpr (RAGGED) __builtin_memcpy(v, vs[T], W * 4);
+        else __builtin_memcpy(v, rd + T * RPI * PITCH_E, W * 4);
         const int m = row0 + 32 * I + T * RPI + lane / LPR;
         const size_t o = (size_t)m * LDD + n;
         if constexpr (RAGGED) {
@@ -244,7 +273,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
         out_t dv[W];
         static_for<W>([&](auto e_c) {
           constexpr int E = decltype(e_c)::value;
-          dv[E] = epilogue<TYPES>(v[E], g.alpha, g.beta, &cv[T][E]);
+          dv[E] = epilogue<TYPES>(v[E], g.alpha, beta_e, &cv[T][E]);
         });
         if (g.store_hint & 1) {   // non-temporal: see mfma_store_hint
           if constexpr (WB == 16) {
@@ -284,7 +313,7 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
             constexpr int C = decltype(c_c)::value;
             const int nn = col0 + C * 64 + lane;
             if (m < M && nn < N && (C < NC - 1 || has_col))
-              g.D[(size_t)m * LDD + nn] = epilogue<TYPES>(v[R][C], g.alpha, g.beta, g.C + (size_t)m * LDC + nn);
+              g.D[(size_t)m * LDD + nn] = epilogue<TYPES>(v[R][C], g.alpha, beta_e, g.C + (size_t)m * LDC + nn);
           });
         });
       }
@@ -295,6 +324,17 @@ __device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g,
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
   });
+}
+template <int TYPES, int FM, int FN, bool RAGGED = false, int BLK = 32, bool TRANSPOSED = false, bool BY4 = false, class Acc,
+          int AM, int AN>
+__device__ __forceinline__ void store_accumulators_lds(const GemmArgs<TYPES>& g, Acc (&acc)[AM][AN], int row0, int col0,
+                                                       int lane, char* region) {
+  if constexpr (RAGGED) {
+    if (g.beta != 0) store_accumulators_lds_impl<1, TYPES, FM, FN, RAGGED, BLK, TRANSPOSED, BY4>(g, acc, row0, col0, lane, region);
+    else store_accumulators_lds_impl<0, TYPES, FM, FN, RAGGED, BLK, TRANSPOSED, BY4>(g, acc, row0, col0, lane, region);
+  } else {
+    store_accumulators_lds_impl<2, TYPES, FM, FN, RAGGED, BLK, TRANSPOSED, BY4>(g, acc, row0, col0, lane, region);
+  }
 }
 template <int FN> constexpr int epilogue_region_bytes() { return 32 * (FN * 32 * 4 + 16); }
 
