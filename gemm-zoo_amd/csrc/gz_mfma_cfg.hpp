@@ -313,7 +313,11 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // 1024 34.1 / 37.2, 34.8 / 35.6; 8000 x 8192 x 2048 218.6 / 240.9, 222.6 / 242.0; fp16 4095 x 4096 x 1024
       // 34.3 / 33.8, 35.1 / 32.4; 8000 x 8192 x 2048 219.5 / 230.7, 231.6 / 226.6; int8 8000 x 8000 x 8192 379 / 414,
       // 402 / 420.)
-      eight = !a_rows || under_a_round || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
+      // (Below one round with a ragged M or N and a 32-bit output the estimate decides as well: us, four / eight waves,
+      // bf16 -> f32 row/col 3000^2 x 4096 70.8 / 76.4, 4000 x 3000 x 2048 48.1 / 53.9, 8000 x 1000 x 4096 76.3 / 79.3,
+      // int8 3000 x 4096 x 2048 28.6 / 31.1; a 16-bit output stays on eight, bf16 -> bf16 3000 x 4096 x 2048 47.4 / 45.3.)
+      const bool ragged = M % 256 != 0 || N % 256 != 0;
+      eight = !a_rows || (under_a_round && (!ragged || out16)) || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
     }
     if (eight) *out = kMfmaCfgs[MFMA_CFG_RING_W8];
   }
