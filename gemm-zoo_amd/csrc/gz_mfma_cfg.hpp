@@ -165,7 +165,10 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
                         (cls == MFMA_SHAPE_WHOLE || (cls == MFMA_SHAPE_RAGGED_MN && i == 0));
     // (128 x 128 beyond four rounds: each further round costs a little more, 6144^2 x 6144 = 9 rounds measured
     // 478 us against 457 for three rounds of 256 x 256)
-    double shape_cost = i == 0 ? (double)rounds : i == 1 ? 0.75 * rounds
+    // (256 x 128 up to one round where every tile has to run on the register-staged kernel - a ragged K, unaligned
+    // lines -: 0.62.  1000 x 8000 x 4000 row/row, 252 tiles against
+    // 504 of 128 x 128, us: bf16 76 / 82, int8 46 / 50, fp16 79 / 86; 8000 x 1000 x 4096 e4m3 47 / 50)
+    double shape_cost = i == 0 ? (double)rounds : i == 1 ? (tiles <= num_cus && cls == MFMA_SHAPE_GENERAL ? 0.62 : 0.75 * rounds)
                                      : 0.40 + 0.27 * rounds + 0.035 * (rounds > 4 ? rounds - 4 : 0);
     const bool f32 = types == GZ_F32F32F32;
     // The register-staged kernel has no second launch for a last round that is mostly empty, but such a round costs
@@ -231,6 +234,9 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
         const double nslab = (double)K * in_size / MFMA_SLAB_BYTES;
         double kf = (8.0 + 1.03 * nslab) / (16.7 + 0.91 * nslab) / 0.987;
         shape_cost *= kf < 0.88 ? 0.88 : kf > 1.06 ? 1.06 : kf;
+        // (and 0.94 of that since the ragged epilogue no longer waits for its own stores: 504 - 512 tiles against
+        // 128 of 256 x 256, K = 4096, us: 8000 x 1000 75.9 / 78.2, 2000 x 4000 73.2 / 74.7; K = 2048 38.3 / 40.8)
+        shape_cost *= 0.94;
       }
       fitted128 = true;
     }
@@ -313,11 +319,12 @@ inline double mfma_choose(int types, int M, int N, int K, int layoutA, int layou
       // 1024 34.1 / 37.2, 34.8 / 35.6; 8000 x 8192 x 2048 218.6 / 240.9, 222.6 / 242.0; fp16 4095 x 4096 x 1024
       // 34.3 / 33.8, 35.1 / 32.4; 8000 x 8192 x 2048 219.5 / 230.7, 231.6 / 226.6; int8 8000 x 8000 x 8192 379 / 414,
       // 402 / 420.)
-      // (Below one round with a ragged M or N and a 32-bit output the estimate decides as well: us, four / eight waves,
+      // (Below one round with a ragged M or N, a K-contiguous B and a 32-bit output the estimate decides as well (a
+      // row-major B stays on eight: 2000 x 4000 x 4096 75.2 / 71.0): us, four / eight waves,
       // bf16 -> f32 row/col 3000^2 x 4096 70.8 / 76.4, 4000 x 3000 x 2048 48.1 / 53.9, 8000 x 1000 x 4096 76.3 / 79.3,
       // int8 3000 x 4096 x 2048 28.6 / 31.1; a 16-bit output stays on eight, bf16 -> bf16 3000 x 4096 x 2048 47.4 / 45.3.)
       const bool ragged = M % 256 != 0 || N % 256 != 0;
-      eight = !a_rows || (under_a_round && (!ragged || out16)) || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
+      eight = !a_rows || (under_a_round && (!ragged || out16 || !b_cols)) || fixed8 + slope8 * nslab < fixed4 + slope4 * nslab;
     }
     if (eight) *out = kMfmaCfgs[MFMA_CFG_RING_W8];
   }
