@@ -90,6 +90,11 @@ def test_plan_headline_configs(capi):
     # int8 consumes 128 k per slab
     p = capi.plan(capi.S8S8S32, 8192, 8192, 8192, 0, 1)
     assert (p.rung, p.tile_k, p.grid) == (capi.RUNG_MFMA, 128, 256)   # 1024 tiles, one persistent work-group per CU
+    # ragged M and N on the same kernel: persistent too (32 x 32 tiles, the last row and column of them clamped), and
+    # the wave estimate decides as for whole tiles (a K-contiguous B and a long K: four waves)
+    p = capi.plan(capi.S8S8S32, 8000, 8000, 8192, 0, 1)
+    assert (p.variant, p.tile_m, p.tile_n, p.threads, p.grid) == (5, 256, 256, 256, 256)
+    assert capi.plan(capi.S8S8S32, 8000, 8000, 8192, 0, 1, capi.RUNG_MFMA, 9).grid == 1024   # one work-group per tile
     # ragged fp16 problem: ceil-div grid, only 2-byte aligned lines
     p = capi.plan(capi.F16F16F16, 4095, 4097, 1023, 0, 0)
     # the one column past 4096 runs as a second launch: dot products, one wave per row, sixteen rows per work-group
